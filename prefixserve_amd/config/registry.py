@@ -1,6 +1,6 @@
 """One registry from an architecture's name to its configuration class and model builder.
 
-``config.json["architectures"][0]`` picks the entry; the entry's configuration class
+``config.json["architectures"][0]`` (or its ``"architecture"``, a plain name) picks the entry; the entry's configuration class
 parses the architecture's own keys and its builder turns the typed configuration into a
 ``ModelSpec``. An unknown name is an error that lists what is registered.
 """
@@ -41,6 +41,8 @@ def registered_architectures() -> list[str]:
 
 def architecture_of(raw: Mapping[str, Any]) -> Architecture:
     archs = raw.get("architectures")
+    if isinstance(raw.get("architecture"), str) and not archs:
+        archs = [raw["architecture"]]            # files that name their one architecture in the singular
     if not archs or not isinstance(archs, list):
         raise UnknownArchitectureError(
             f"config.json has no 'architectures' entry; registered: {registered_architectures()}")

@@ -33,6 +33,35 @@ int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, in
 int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
                          const int32_t* positions, const float* table, void* kv, const int32_t* write_slot);
 
+// The norm behind the sum: x = alpha * residual + delta (delta as for psamd_add_rmsnorm, or NULL),
+// y = weight * rmsnorm(x) in float; residual[r] = y[r] and, if out is given, out[r] = y[r] in act_dtype.
+int psamd_scaled_add_rmsnorm(void* stream, float* residual, float alpha, const void* delta, int delta_dtype,
+                             int n_partials, int64_t partial_stride, const void* weight, int weight_dtype, float eps,
+                             void* out, int act_dtype, int64_t rows, int hidden);
+
+// out[i] = in[i] in act_dtype.
+int psamd_to_activation(void* stream, const float* in, void* out, int act_dtype, int64_t n);
+
+// psamd_rope_kv_append with a unit norm behind the rotation: every q and k head is divided by
+// sqrt(sum of its squares / norm_dim + eps) (norm_dim 0: no norm; norm_dim < head_dim: the rest of
+// the head's slots hold zeros). hkv may be 0: rows of queries alone.
+int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                              const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
+                              const int32_t* write_slot);
+
+// Mixture of experts. Router: z = x w_router^T in float (x in x_dtype, w_router float [E, K]), score =
+// sigmoid(z); chosen[t, :] = the top largest scores' experts (lower index among equals, largest
+// first), weight[t, :] = those scores.
+int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_router, int32_t* chosen, float* weight,
+                    int64_t tokens, int K, int experts, int top);
+// Experts, one (token, choice) pair at a time: h = weight[t, j] * x[t]; g = min(gate h, limit), u =
+// clamp(up h, -limit, limit); act[t * top + j] = g * sigmoid(gate_alpha * g) * (u + up_shift);
+// out[j][t] = down act (float). w_gate_up is [E, 2F, K] (gate rows, then up rows), w_down [E, K, F].
+int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, const float* weight,
+                           const void* w_gate_up, const void* w_down, void* act, float* out, int dtype,
+                           int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
+                           float up_shift);
+
 // out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
                  int64_t M, int N, int K);

@@ -369,6 +369,139 @@ __global__ __launch_bounds__(256) void rope_kv_append_vec_kernel(bf16_t* __restr
   }
 }
 
+// ------------------------------------------------------------------ norm behind the sum
+
+// One block per row: x = alpha * residual + sum of the delta slices, y = weight * x *
+// rsqrt(mean(x^2) + eps), all in float; y becomes the new residual row and, if `out` is given,
+// is also written in the activation type (the copy the next product reads). Rows up to
+// kCache * kThreads wide stay in registers between the two passes; wider ones pass through
+// the residual row itself.
+template <typename A, typename DT, int kThreads, int kCache>
+__global__ __launch_bounds__(kThreads) void scaled_add_rmsnorm_kernel(
+    float* __restrict__ residual, float alpha, const DT* __restrict__ delta, int n_partials, int64_t partial_stride,
+    const void* __restrict__ weight, int weight_dtype, float eps, A* __restrict__ out, int hidden) {
+  __shared__ float scratch[kThreads / kWave];
+  float* r = residual + static_cast<int64_t>(blockIdx.x) * hidden;
+  const DT* d0 = delta != nullptr ? delta + static_cast<int64_t>(blockIdx.x) * hidden : nullptr;
+  A* o = out != nullptr ? out + static_cast<int64_t>(blockIdx.x) * hidden : nullptr;
+  const int np = delta != nullptr ? n_partials : 0;
+  if (hidden <= kCache * kThreads) {
+    float v[kCache];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      const int i = static_cast<int>(threadIdx.x) + j * kThreads;
+      const int ic = min(i, hidden - 1);
+      float x = alpha * r[ic];
+      for (int p = 0; p < np; ++p) x += to_float<DT>(d0[p * partial_stride + ic]);
+      v[j] = x;
+      ss += i < hidden ? x * x : 0.f;
+    }
+    ss = block_sum(ss, scratch, kThreads / kWave);
+    const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int j = 0; j < kCache; ++j) {
+      const int i = static_cast<int>(threadIdx.x) + j * kThreads;
+      if (i < hidden) {
+        const float y = load_as_float(weight, weight_dtype, i) * (v[j] * inv);
+        r[i] = y;
+        if (o != nullptr) o[i] = from_float<A>(y);
+      }
+    }
+    return;
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    float x = alpha * r[i];
+    for (int p = 0; p < np; ++p) x += to_float<DT>(d0[p * partial_stride + i]);
+    r[i] = x;
+    ss += x * x;
+  }
+  ss = block_sum(ss, scratch, kThreads / kWave);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    const float y = load_as_float(weight, weight_dtype, i) * (r[i] * inv);
+    r[i] = y;
+    if (o != nullptr) o[i] = from_float<A>(y);
+  }
+}
+
+// out[i] = A(in[i]): the float32 stream in the activation type.
+template <typename A>
+__global__ void to_activation_kernel(const float* __restrict__ in, A* __restrict__ out, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    out[i] = from_float<A>(in[i]);
+}
+
+// ------------------------------------------------------------------ rope + unit norm + kv append
+
+// One wave per (token, head) of a row [hq q heads | hkv k heads | hkv v heads] x d. A q or k head
+// is rotated (pair (i, i + d/2), table [pos][i] = (cos, sin); NULL: not rotated), then, with
+// norm_dim > 0, divided by sqrt(sum of squares / norm_dim + eps): the root mean square over the
+// norm_dim dimensions that are the head's own when the rest of its d slots hold zeros. The
+// result goes back into the row and, for a k head, to its page as a [16, d] row; a v head goes
+// to the page's second half transposed, [d, 16]. hkv may be 0 (a row of queries alone).
+template <typename A>
+__global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
+    A* __restrict__ qkv, int hq, int hkv, int d, const int32_t* __restrict__ positions,
+    const float2* __restrict__ table, int norm_dim, float eps, A* __restrict__ kv,
+    const int32_t* __restrict__ write_slot) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int head = static_cast<int>(blockIdx.y) * 4 + static_cast<int>(threadIdx.x >> 6);
+  if (head >= hq + 2 * hkv) return;
+  const int half = d >> 1;
+  A* row = qkv + t * (static_cast<int64_t>(hq + 2 * hkv) * d) + static_cast<int64_t>(head) * d;
+  int64_t page = 0;
+  int off = 0;
+  if (kv != nullptr) {
+    const int slot = write_slot[t];
+    page = slot / kPage;
+    off = slot % kPage;
+  }
+  const int64_t page_elems = 2LL * hkv * kPage * d;
+  if (head < hq + hkv) {
+    const int pos = positions[t];
+    float a[2], b[2];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i = lane + j * kWave;
+      a[j] = b[j] = 0.f;
+      if (i < half) {
+        const float u = to_float<A>(row[i]), v = to_float<A>(row[i + half]);
+        float2 cs = float2{1.f, 0.f};
+        if (table != nullptr) cs = table[static_cast<int64_t>(pos) * half + i];
+        a[j] = u * cs.x - v * cs.y;
+        b[j] = v * cs.x + u * cs.y;
+        ss += a[j] * a[j] + b[j] * b[j];
+      }
+    }
+    float inv = 1.f;
+    if (norm_dim > 0) inv = rsqrtf(wave_sum(ss) / static_cast<float>(norm_dim) + eps);
+    A* dst = (kv != nullptr && head >= hq)
+                 ? kv + page * page_elems + (static_cast<int64_t>(head - hq) * kPage + off) * d : nullptr;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i = lane + j * kWave;
+      if (i < half) {
+        const A lo = from_float<A>(a[j] * inv), hi = from_float<A>(b[j] * inv);
+        row[i] = lo;
+        row[i + half] = hi;
+        if (dst != nullptr) {
+          dst[i] = lo;
+          dst[i + half] = hi;
+        }
+      }
+    }
+  } else if (kv != nullptr) {
+    const int vh = head - hq - hkv;
+    A* vpage = kv + page * page_elems + static_cast<int64_t>(hkv) * kPage * d + off;
+    for (int c = lane; c < d; c += kWave) vpage[(static_cast<int64_t>(vh) * d + c) * kPage] = row[c];
+  }
+}
+
 }  // namespace psamd
 
 using namespace psamd;
@@ -484,6 +617,72 @@ int psamd_rope_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens,
     return fail("psamd_rope_kv_append: activation dtype must be float32 or bfloat16");
   }
   return check_launch("psamd_rope_kv_append");
+}
+
+int psamd_scaled_add_rmsnorm(void* stream, float* residual, float alpha, const void* delta, int delta_dtype,
+                             int n_partials, int64_t partial_stride, const void* weight, int weight_dtype, float eps,
+                             void* out, int act_dtype, int64_t rows, int hidden) {
+  PSAMD_REQUIRE(rows >= 0 && hidden > 0, "bad sizes");
+  PSAMD_REQUIRE(weight_dtype == kF32 || weight_dtype == kBF16, "weight dtype must be float32 or bfloat16");
+  PSAMD_REQUIRE(delta == nullptr || delta_dtype == kF32 || delta_dtype == kBF16, "delta dtype");
+  PSAMD_REQUIRE(delta == nullptr || (n_partials >= 1 && (n_partials == 1 || delta_dtype == kF32)),
+                "partial sums must be float32");
+  PSAMD_REQUIRE(out == nullptr || act_dtype == kF32 || act_dtype == kBF16, "activation dtype");
+  if (rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  constexpr int kThreads = 256, kCache = 16;
+  const dim3 grid(static_cast<unsigned>(rows)), block(kThreads);
+#define PSAMD_POSTNORM(A_, D_)                                                                              \
+  scaled_add_rmsnorm_kernel<A_, D_, kThreads, kCache><<<grid, block, 0, s>>>(                               \
+      residual, alpha, static_cast<const D_*>(delta), n_partials, partial_stride, weight, weight_dtype, eps, \
+      static_cast<A_*>(out), hidden)
+  const bool delta_f32 = delta == nullptr || delta_dtype == kF32;
+  if (out != nullptr && act_dtype == kBF16) {
+    if (delta_f32) PSAMD_POSTNORM(bf16_t, float); else PSAMD_POSTNORM(bf16_t, bf16_t);
+  } else {
+    if (delta_f32) PSAMD_POSTNORM(float, float); else PSAMD_POSTNORM(float, bf16_t);
+  }
+#undef PSAMD_POSTNORM
+  return check_launch("psamd_scaled_add_rmsnorm");
+}
+
+int psamd_to_activation(void* stream, const float* in, void* out, int act_dtype, int64_t n) {
+  PSAMD_REQUIRE(n >= 0, "bad size");
+  if (n == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
+  if (act_dtype == kBF16) {
+    to_activation_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(in, static_cast<bf16_t*>(out), n);
+  } else if (act_dtype == kF32) {
+    to_activation_kernel<float><<<dim3(blocks), dim3(256), 0, s>>>(in, static_cast<float*>(out), n);
+  } else {
+    return fail("psamd_to_activation: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_to_activation");
+}
+
+int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                              const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
+                              const int32_t* write_slot) {
+  PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv >= 0, "bad sizes");
+  PSAMD_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256, "head_dim must be even and at most 256");
+  PSAMD_REQUIRE(norm_dim >= 0 && norm_dim <= head_dim, "norm_dim must be in [0, head_dim]");
+  PSAMD_REQUIRE(kv == nullptr || (write_slot != nullptr && hkv > 0), "a cache needs write slots and kv heads");
+  PSAMD_REQUIRE(tokens <= 2147483647LL && ceil_div(hq + 2 * hkv, 4) <= 65535, "too large for one launch");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float2* tab = reinterpret_cast<const float2*>(table);
+  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(ceil_div(hq + 2 * hkv, 4)));
+  if (act_dtype == kBF16) {
+    rope_norm_kv_append_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim, positions,
+                                                                 tab, norm_dim, eps, static_cast<bf16_t*>(kv), write_slot);
+  } else if (act_dtype == kF32) {
+    rope_norm_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<float*>(qkv), hq, hkv, head_dim, positions,
+                                                                tab, norm_dim, eps, static_cast<float*>(kv), write_slot);
+  } else {
+    return fail("psamd_rope_norm_kv_append: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_rope_norm_kv_append");
 }
 
 }  // extern "C"

@@ -83,6 +83,9 @@ class StepContext:
     # The step's residual stream (float32 [T, hidden]), set by the model before the layers run: a
     # part may add its output into it itself instead of handing back what is to be added.
     residual: Any = None
+    # The stream's copy in the activation dtype when a block has just written one beside it
+    # (a norm behind the sum does): the next block's sub-layer reads it instead of converting.
+    stream_copy: Any = None
 
 
 class StepPacker:

@@ -69,6 +69,11 @@ _SIGNATURES = {
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
+    "psamd_scaled_add_rmsnorm": [_vp, _vp, _f32, _vp, _i32, _i32, _i64, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
+    "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
+    "psamd_rope_norm_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp],
+    "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
 }
 
 
@@ -245,6 +250,25 @@ class HipOps:
                                             rows.data_ptr(), weight.data_ptr(), _code(weight.dtype), eps,
                                             out.data_ptr(), _code(out.dtype), s, h))
 
+    def scaled_add_rmsnorm(self, residual, delta, alpha: float, weight, eps: float, out) -> None:
+        """The norm behind the sum: residual <- weight * rmsnorm(alpha * residual + delta), in 32-bit and
+        in place; ``out`` (or None) receives the same rows in the activation dtype."""
+        t, h = residual.shape
+        self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "scaled_add_rmsnorm: residual must be float32")
+        self._need(weight.numel() == h and weight.is_contiguous(), "scaled_add_rmsnorm: weight size")
+        if out is not None:
+            self._need(out.shape == (t, h) and out.is_contiguous(), "scaled_add_rmsnorm: bad output shape")
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, out.dtype if out is not None else torch.float32)
+        self._ok(self.lib.psamd_scaled_add_rmsnorm(self._stream(), residual.data_ptr(), float(alpha), dptr, dcode, slices,
+                                                   stride, weight.data_ptr(), _code(weight.dtype), float(eps), _ptr(out),
+                                                   _code(out.dtype) if out is not None else _F32, t, h))
+
+    def to_activation(self, src, out) -> None:
+        """out = src (float32) in out's dtype."""
+        self._need(src.dtype == torch.float32 and src.is_contiguous() and out.is_contiguous() and src.shape == out.shape,
+                   "to_activation: a float32 tensor and an output of its shape")
+        self._ok(self.lib.psamd_to_activation(self._stream(), src.data_ptr(), out.data_ptr(), _code(out.dtype), src.numel()))
+
     def swiglu(self, gate_up, out) -> None:
         t, inter = out.shape
         self._need(gate_up.shape == (t, 2 * inter) and gate_up.dtype == out.dtype, "swiglu: shapes")
@@ -264,6 +288,27 @@ class HipOps:
         self._ok(self.lib.psamd_rope_kv_append(self._stream(), qkv.data_ptr(), _code(qkv.dtype), t, hq, hkv, d,
                                                positions.data_ptr(), _ptr(table), _ptr(kv),
                                                None if kv is None else write_slot.data_ptr()))
+
+    def rope_norm_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot, norm_dim: int,
+                            norm_eps: float) -> None:
+        """``rope_kv_append`` with every q and k head divided, behind the rotation, by the root mean
+        square over its ``norm_dim`` own dimensions (0: no norm; the head's other slots hold zeros).
+        ``hkv`` may be 0: rows of queries alone, nothing written to pages."""
+        t = qkv.shape[0]
+        self._need(qkv.shape[1] == (hq + 2 * hkv) * d and qkv.is_contiguous(), "rope_norm_kv_append: qkv shape")
+        self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_norm_kv_append: positions")
+        self._need(0 <= norm_dim <= d and d % 2 == 0 and d <= 256, "rope_norm_kv_append: head sizes")
+        if table is not None:
+            self._need(table.dtype == torch.float32 and table.shape[1:] == (d // 2, 2) and table.is_contiguous(),
+                       "rope_norm_kv_append: table must be float32 [positions, D/2, 2]")
+            self._need(table.shape[0] >= 1, "rope_norm_kv_append: empty table")
+        if kv is not None:
+            self._need(hkv > 0 and kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                       "rope_norm_kv_append: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+            self._need(write_slot.dtype == torch.int32 and write_slot.numel() == t, "rope_norm_kv_append: write slots")
+        self._ok(self.lib.psamd_rope_norm_kv_append(self._stream(), qkv.data_ptr(), _code(qkv.dtype), t, hq, hkv, d,
+                                                    positions.data_ptr(), _ptr(table), int(norm_dim), float(norm_eps),
+                                                    _ptr(kv), None if kv is None else write_slot.data_ptr()))
 
     def qkv_rope_append(self, x, w_qkv, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot) -> None:
         """qkv = x @ w_qkv^T, q and k rotated, k and v written to their pages. One kernel for a
@@ -422,6 +467,42 @@ class HipOps:
         gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
         self.linear(x, w_gate_up, gu)
         self.swiglu(gu, out)
+
+    # ------------------------------------------------------------------ experts
+
+    def moe_route(self, x, w_router, chosen, weight) -> None:
+        """chosen[t, :], weight[t, :] = the experts with the largest sigmoid(x[t] . w_router[e]) and
+        those scores, largest first, the lower index among equals; scores in 32-bit."""
+        t, k = x.shape
+        e, top = w_router.shape[0], chosen.shape[1]
+        self._need(x.is_contiguous() and w_router.dtype == torch.float32 and w_router.is_contiguous()
+                   and w_router.shape[1] == k, "moe_route: x [T, K], router float32 [E, K]")
+        self._need(chosen.dtype == torch.int32 and weight.dtype == torch.float32 and chosen.shape == (t, top)
+                   and weight.shape == (t, top) and chosen.is_contiguous() and weight.is_contiguous() and 1 <= top <= e,
+                   "moe_route: outputs must be int32 and float32 [T, top]")
+        self._ok(self.lib.psamd_moe_route(self._stream(), x.data_ptr(), _code(x.dtype), w_router.data_ptr(),
+                                          chosen.data_ptr(), weight.data_ptr(), t, k, e, top))
+
+    def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha: float, limit: float,
+                    up_shift: float) -> None:
+        """out[j, t] = down_e(act_e(weight[t, j] * x[t])) for e = chosen[t, j], as float32 slices [top, T, K];
+        ``act`` [T * top, F] is scratch in the activation dtype."""
+        t, k = x.shape
+        top = chosen.shape[1]
+        e, f2, _ = w_gate_up.shape
+        f = f2 // 2
+        self._need(w_gate_up.shape == (e, 2 * f, k) and w_down.shape == (e, k, f) and w_gate_up.is_contiguous()
+                   and w_down.is_contiguous() and w_gate_up.dtype == x.dtype and w_down.dtype == x.dtype,
+                   "moe_experts: weights must be [E, 2F, K] and [E, K, F] in the activation dtype")
+        self._need(x.is_contiguous() and chosen.shape == (t, top) and weight.shape == (t, top) and chosen.dtype == torch.int32
+                   and weight.dtype == torch.float32 and chosen.is_contiguous() and weight.is_contiguous(),
+                   "moe_experts: the router's outputs")
+        self._need(act.shape == (t * top, f) and act.dtype == x.dtype and act.is_contiguous(), "moe_experts: act scratch")
+        self._need(out.shape == (top, t, k) and out.dtype == torch.float32 and out.is_contiguous(), "moe_experts: output slices")
+        self._ok(self.lib.psamd_moe_experts_rows(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
+                                                 w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(), out.data_ptr(),
+                                                 _code(x.dtype), t, k, f, e, top, float(gate_alpha), float(limit),
+                                                 float(up_shift)))
 
     # --------------------------------------------------------------- attention
 

@@ -1,3 +1,4 @@
 """Architectures known to the registry. Importing this package registers them."""
 
 from . import llama  # noqa: F401
+from . import radivik  # noqa: F401

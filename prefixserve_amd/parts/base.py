@@ -159,6 +159,13 @@ class Norm(Part):
         """The same for the selected rows only; ``residual`` is left as it is."""
         raise NotImplementedError
 
+    def norm_of_sum(self, residual: torch.Tensor, delta: torch.Tensor | None, alpha: float,
+                    out_name: str) -> torch.Tensor:
+        """The norm behind the sum: residual (float32 [T,H], in place) <- norm(alpha * residual +
+        delta), all of it in 32-bit; ``delta`` as for ``add_norm``. Returns the new stream in the
+        activation dtype (the stream itself when that is float32): what the next sub-layer reads."""
+        raise NotImplementedError
+
 
 class PositionEncoding(Part):
     """Position information applied to queries and keys before attention."""
@@ -171,9 +178,13 @@ class RotaryTable(PositionEncoding):
     """A position encoding that rotates the pairs (i, i + D/2) of every query and key head by
     an angle that depends on the position and on i. It has ``head_dim`` and, once ``prepare``
     ran, ``table``: float32 ``[max_position, head_dim / 2, 2]`` = (cos, sin) on the device.
-    How the angles come about is the subclass's business; attention only reads the table."""
+    How the angles come about is the subclass's business; attention only reads the table.
+    ``rotary_dim`` (None: the whole head) says that only the model's first ``rotary_dim``
+    dimensions of a head rotate, partners ``rotary_dim / 2`` apart: the table's other pair
+    slots are the identity and the mixer puts the partners into slots ``head_dim / 2`` apart."""
 
     head_dim: int
+    rotary_dim: int | None = None
     table: torch.Tensor | None = None
 
 

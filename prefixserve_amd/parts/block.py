@@ -33,6 +33,7 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
                 state: torch.Tensor | None, writes_cache: bool) -> torch.Tensor:
+        ctx.stream_copy = None               # the stream moves on without its activation-dtype copy
         if self.mixer.takes_normed_rows:
             x = self.mixer_norm.add_norm(residual, pending, "block.x", lazy=True)
         else:
@@ -45,4 +46,46 @@ class PreNormBlock:
         return self.feed_forward.forward(x, ctx)
 
 
+class PostNormBlock:
+    """The norm behind the sum: x <- norm1(alpha x + mixer(x)), then, when the layer has a
+    feed-forward, x <- norm2(alpha x + feed_forward(x)). The sub-layers read the stream itself,
+    which is a normalized vector from the first layer's first norm on; ``alpha`` is the factor
+    on the stream in front of each sum (1: the plain arrangement). Sum, statistics and the
+    stream are float32; beside the stream the norm writes its copy in the activation dtype
+    for the next sub-layer's products (``ctx.stream_copy``, so that the next block of this
+    kind does not convert again). ``feed_forward`` None: the second half does not exist."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm,
+                 feed_forward_norm: Norm | None, alpha: float = 1.0) -> None:
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.alpha = float(alpha)
+
+    def parts(self) -> list[Part]:
+        both = [self.mixer_norm, self.mixer]
+        return both + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
+
+    def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
+                state: torch.Tensor | None, writes_cache: bool) -> None:
+        rt = self.mixer_norm.rt
+        if pending is not None:
+            # A sub-layer in front left its output to be added: the norm's fused sum does that
+            # (its normalized output is not wanted here).
+            self.mixer_norm.add_norm(residual, pending, "block.x")
+            ctx.stream_copy = None
+        kept, ctx.residual = ctx.residual, None   # the sub-layers hand their output back: it is normalized with the stream
+        x = residual if rt.dtype == torch.float32 else getattr(ctx, "stream_copy", None)
+        if x is None:
+            x = rt.workspace.get("block.x", tuple(residual.shape), rt.dtype)
+            rt.ops.to_activation(residual, x)
+        mixed = self.mixer.forward(x, ctx, cache, state, writes_cache)
+        x = self.mixer_norm.norm_of_sum(residual, mixed, self.alpha, "block.x")
+        if self.feed_forward is not None:
+            x = self.feed_forward_norm.norm_of_sum(residual, self.feed_forward.forward(x, ctx), self.alpha, "block.x")
+        ctx.stream_copy = x
+        ctx.residual = kept
+        return None
+
+
 register_block("prenorm", PreNormBlock)
+register_block("postnorm", PostNormBlock)

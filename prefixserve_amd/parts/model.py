@@ -11,6 +11,7 @@ import torch
 from . import attention as _attention  # noqa: F401  (registers the built-in parts)
 from . import block as _block  # noqa: F401
 from . import mlp as _mlp  # noqa: F401
+from . import moe as _moe  # noqa: F401
 from . import norm as _norm  # noqa: F401
 from . import rope as _rope  # noqa: F401
 from .base import CacheNeed, Part, Runtime, StateNeed, WeightWant, make
@@ -29,12 +30,15 @@ class DecoderModel:
         for layer in spec.layers:
             h = spec.hidden_size
             mixer = make("mixer", layer.mixer.kind, hidden_size=h, positions=self.positions, **layer.mixer.params)
-            ff = make("feed_forward", layer.feed_forward.kind, hidden_size=h, **layer.feed_forward.params)
+            ff = n2 = None
+            if layer.feed_forward is not None:
+                ff = make("feed_forward", layer.feed_forward.kind, hidden_size=h, **layer.feed_forward.params)
             n1 = make("norm", layer.mixer_norm.kind, hidden_size=h, **layer.mixer_norm.params)
-            n2 = make("norm", layer.feed_forward_norm.kind, hidden_size=h, **layer.feed_forward_norm.params)
+            if layer.feed_forward_norm is not None:
+                n2 = make("norm", layer.feed_forward_norm.kind, hidden_size=h, **layer.feed_forward_norm.params)
             extra = {name: make("norm", ps.kind, hidden_size=h, **ps.params) for name, ps in layer.extra_norms.items()}
             self.blocks.append(make("block", layer.block, mixer=mixer, feed_forward=ff, mixer_norm=n1,
-                                    feed_forward_norm=n2, **extra))
+                                    feed_forward_norm=n2, **extra, **layer.block_params))
         self.final_norm = make("norm", spec.final_norm.kind, hidden_size=spec.hidden_size, **spec.final_norm.params)
         sizes = dict(hidden_size=spec.hidden_size, vocab_size=spec.vocab_size)
         self.embedding_transforms = [make("transform", ps.kind, **sizes, **ps.params) for ps in spec.embedding_transforms]
@@ -134,6 +138,7 @@ class DecoderModel:
             for tr in self.embedding_transforms:
                 tr.apply(residual, ctx, None)
             ctx.residual = residual
+            ctx.stream_copy = None           # a context may be stepped twice (a graph's eager run, then its capture)
             pending = None
             for i, run in enumerate(s.order):
                 pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),

@@ -56,4 +56,12 @@ class RMSNorm(Norm):
         return out
 
 
+    def norm_of_sum(self, residual: torch.Tensor, delta: torch.Tensor | None, alpha: float,
+                    out_name: str) -> torch.Tensor:
+        rt = self.rt
+        out = None if rt.dtype == torch.float32 else rt.workspace.get(out_name, tuple(residual.shape), rt.dtype)
+        rt.ops.scaled_add_rmsnorm(residual, delta, float(alpha), self.weight, self.eps, out)
+        return residual if out is None else out
+
+
 register_norm("rmsnorm", RMSNorm)

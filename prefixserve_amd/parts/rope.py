@@ -61,4 +61,57 @@ class RotaryEmbedding(RotaryTable):
         self.max_position = int(max_position)
 
 
+def yarn_inv_freq(rotary_dim: int, base: float, scaling: Mapping[str, Any] | None) -> tuple[torch.Tensor, float]:
+    """(float64 frequencies f_i = base^(-2i/r), i < r/2, after YaRN scaling; the factor on cos and sin).
+
+    ``scaling`` = (factor s, original length L, fast, slow): a wave that makes t turns over L
+    sits at dimension dim(t) = r ln(L / (2 pi t)) / (2 ln base). Below lo = floor(dim(fast)) a
+    frequency is kept, above hi = ceil(dim(slow)) it is divided by s, in between the share of
+    the divided one rises linearly (lo and hi are kept inside [0, r - 1]; a span of zero counts
+    as 0.001). Cosine and sine are multiplied by 0.1 ln(s) + 1."""
+    i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+    f = torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / rotary_dim)
+    if scaling is None:
+        return f, 1.0
+    s, orig = float(scaling["factor"]), float(scaling["original"])
+
+    def dim_of(turns: float) -> float:
+        return rotary_dim * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+    lo = max(math.floor(dim_of(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(dim_of(float(scaling["slow"]))), rotary_dim - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return f / s * ramp + f * (1.0 - ramp), 0.1 * math.log(s) + 1.0
+
+
+class YarnRotary(RotaryTable):
+    """A rotation of the first ``rotary_dim`` dimensions of a head only, with YaRN-scaled
+    frequencies and its factor on cosine and sine. The table has ``head_dim / 2`` pair slots
+    like every ``RotaryTable``: the first ``rotary_dim / 2`` carry the angles, the others are
+    the identity (1, 0), so the kernels that rotate whole heads leave the rest of a head as it
+    is. The mixer lays a head out accordingly (``rotary_dim`` tells it to): the partners
+    (i, i + rotary_dim/2) of the model's layout sit in slots (i, i + head_dim/2).
+    Angles are position x frequency in float64, rounded once to float32 as cos and sin."""
+
+    def __init__(self, head_dim: int, rotary_dim: int, base: float, scaling: Mapping[str, Any] | None = None) -> None:
+        if head_dim % 2 or rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even and at most head_dim {head_dim} (even)")
+        self.head_dim, self.rotary_dim = int(head_dim), int(rotary_dim)
+        self.base = float(base)
+        self.scaling = dict(scaling) if scaling is not None else None
+        self.table: torch.Tensor | None = None
+
+    def prepare(self, max_position: int) -> None:
+        table = torch.zeros((max_position, self.head_dim // 2, 2), dtype=torch.float64)
+        table[:, :, 0] = 1.0
+        if self.rotary_dim:
+            freq, gain = yarn_inv_freq(self.rotary_dim, self.base, self.scaling)
+            angle = torch.outer(torch.arange(max_position, dtype=torch.float64), freq)
+            table[:, : self.rotary_dim // 2, 0] = angle.cos() * gain
+            table[:, : self.rotary_dim // 2, 1] = angle.sin() * gain
+        self.table = table.to(torch.float32).contiguous().to(self.rt.device)
+        self.max_position = int(max_position)
+
+
 register_position("rope", RotaryEmbedding)
+register_position("yarn", YarnRotary)

@@ -27,10 +27,12 @@ class LayerSpec:
 
     prefix: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None        # None: a layer without a feed-forward (for arrangements that take that)
     mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    feed_forward_norm: PartSpec | None
     block: str = "prenorm"
+    # Constants of the arrangement itself (a factor on the stream in front of a sum, say).
+    block_params: Mapping[str, Any] = field(default_factory=dict)
     # Further norms an arrangement other than "prenorm" may want (norms behind the sub-layers,
     # say): built like the two above and handed to the block's factory by these names.
     extra_norms: Mapping[str, PartSpec] = field(default_factory=dict)

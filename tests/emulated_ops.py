@@ -82,6 +82,57 @@ class EmulatedOps:
             kpages[page, :, off, :] = k
             vpages[page, :, :, off] = v
 
+    def normed(self, x, name="normed.x"):
+        return x
+
+    def to_activation(self, src, out) -> None:
+        out.copy_(src.to(out.dtype))
+
+    def scaled_add_rmsnorm(self, residual, delta, alpha, weight, eps, out) -> None:
+        x = residual * alpha
+        if delta is not None:
+            x = x + (delta.float().sum(0) if delta.dim() == 3 else delta.float())
+        y = weight.float() * x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+        residual.copy_(y)
+        if out is not None:
+            out.copy_(y.to(out.dtype))
+
+    def rope_norm_kv_append(self, qkv, hq, hkv, d, positions, table, kv, write_slot, norm_dim, norm_eps) -> None:
+        t = qkv.shape[0]
+        heads = qkv[:, : (hq + hkv) * d].view(t, hq + hkv, d)
+        x = heads.float()
+        if table is not None:
+            cs = table[positions.long()]
+            cos, sin = cs[..., 0][:, None, :], cs[..., 1][:, None, :]
+            x1, x2 = x[..., : d // 2], x[..., d // 2:]
+            x = torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
+        if norm_dim:
+            x = x * torch.rsqrt((x * x).sum(-1, keepdim=True) / norm_dim + norm_eps)
+        heads.copy_(x.to(qkv.dtype))
+        if kv is not None:
+            page, off = (write_slot // PAGE).long(), (write_slot % PAGE).long()
+            kv[:, 0].view(kv.shape[0], hkv, PAGE, d)[page, :, off, :] = heads[:, hq:]
+            kv[:, 1].view(kv.shape[0], hkv, d, PAGE)[page, :, :, off] = qkv[:, (hq + hkv) * d:].view(t, hkv, d)
+
+    def moe_route(self, x, w_router, chosen, weight) -> None:
+        s = torch.sigmoid(x.float() @ w_router.float().T)
+        order = torch.argsort(-s, dim=-1, stable=True)[:, : chosen.shape[1]]
+        chosen.copy_(order.to(torch.int32))
+        weight.copy_(torch.gather(s, 1, order))
+
+    def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha, limit, up_shift) -> None:
+        t, k = chosen.shape
+        f = w_gate_up.shape[1] // 2
+        for i in range(t):
+            for j in range(k):
+                e = int(chosen[i, j])
+                h = x[i].float() * weight[i, j]
+                gu = w_gate_up[e].float() @ h
+                g, u = gu[:f].clamp(max=limit), gu[f:].clamp(-limit, limit)
+                y = (g * torch.sigmoid(gate_alpha * g) * (u + up_shift)).to(act.dtype)
+                act[i * k + j] = y
+                out[j, i] = w_down[e].float() @ y.float()
+
     def expand_kv(self, x, rep):
         """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
         return x.repeat_interleave(rep, dim=1)
