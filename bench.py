@@ -56,6 +56,120 @@ SHAPES = {
 }
 
 
+# Radivik at sizes that resemble real layers, each beside the Llama decoder of equal size: same
+# width, head counts, head size (the size Radivik's pages run with) and vocabulary, and an inner
+# feed-forward size of top x ff, so that a token passes through as many weights in both.
+RADIVIK_SIZES = {
+    # 1B-like: the default shape's width and heads, 32 experts of which 8 make its inner size
+    "w2048-h32x64-e32x1024-top8": dict(width=2048, heads=32, kv_heads=8, dim=64, vdim=64, rot=32, experts=32, ff=1024, top=8),
+    # 8B-like width and head size, 16 experts of which 4 are used; every other layer reads its neighbour's keys
+    "w4096-h32x128-e16x3584-top4": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, rot=64, experts=16, ff=3584, top=4,
+                                        share=True),
+    # a value size larger than the query/key size: the pages run with the larger one
+    "w3072-h24x96v128-e64x512-top8": dict(width=3072, heads=24, kv_heads=8, dim=96, vdim=128, rot=48, experts=64, ff=512, top=8),
+}
+
+
+def radivik_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
+    """(Radivik config.json, the Llama config.json of equal size)."""
+    rot = {"base": 500000.0, "dims": size["rot"], "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
+             "scale": size["dim"] ** -0.5 * 4.0, "rot": rot}
+    mlp = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": size["ff"], "limit": 7.0}}
+    entries = []
+    for i in range(layers):
+        m = dict(mixer)
+        if size.get("share") and i % 2 == 1:
+            m["kv_from"] = i - 1
+        entries.append({"type": "attention", "mixer": m, "mlp": mlp})
+    radivik = {"architecture": "Radivik", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-5}, "postln_alpha": 2.0,
+               "layers": entries}
+    slot = max(size["dim"], size["vdim"])
+    llama = dict(LLAMA_1B, vocab_size=vocab, hidden_size=size["width"], intermediate_size=size["top"] * size["ff"],
+                 num_hidden_layers=layers, num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"],
+                 head_dim=slot, tie_word_embeddings=False)
+    return radivik, llama
+
+
+def compare_designs(args) -> int:
+    """Prefill and decode throughput of Radivik layers beside Llama layers of equal size, through
+    the same runner and step function. One JSON line; the default benchmark is not run."""
+    import numpy as np
+    import torch
+
+    from prefixserve_amd.engine.batch import StepItem
+    from prefixserve_amd.engine.runner import ModelRunner
+    from prefixserve_amd.weights import write_random_model
+
+    rng = np.random.default_rng(0)
+    vocab, layers = 32000, args.layers or 4
+    prompt, batch, context = args.prompt_len, args.batch, args.context
+    sizes = RADIVIK_SIZES if args.compare == "all" else {args.compare: RADIVIK_SIZES[args.compare]}
+    results = {}
+
+    def measure(folder) -> dict:
+        pages_per = -(-context // 16)
+        runner = ModelRunner(folder, dtype=args.dtype, num_blocks=(batch + 1) * pages_per + 8, max_seq_len=context,
+                             max_num_seqs=max(batch, 2), max_prefill_tokens=prompt, use_graphs=not args.no_graphs)
+        groups = len(runner.num_blocks_per_group)
+        tables = [[list(range(b * pages_per, (b + 1) * pages_per)) for _ in range(groups)] for b in range(batch + 1)]
+        toks = rng.integers(0, vocab, prompt)
+
+        def timed(fn, reps: int) -> float:
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps
+
+        whole = lambda: runner.step([StepItem("p", toks, 0, tables[batch], 0, (prompt - 1,))])
+        t_prefill = timed(whole, args.prefill_reps)
+        fill = context - args.steps - args.warmup - 2
+        for b in range(batch):                                  # every request's cache, filled in portions
+            for p0 in range(0, fill, prompt):
+                n = min(prompt, fill - p0)
+                runner.step([StepItem(f"d{b}", rng.integers(0, vocab, n), p0, tables[b], b, ())])
+        pos = [fill]
+
+        def decode():
+            runner.step([StepItem(f"d{b}", (1,), pos[0], tables[b], b, (0,)) for b in range(batch)])
+            pos[0] += 1
+
+        for _ in range(args.warmup):
+            decode()
+        t_decode = timed(decode, args.steps)
+        weights = runner.model.step_weight_bytes()
+        kv = batch * (fill + args.steps / 2) * sum(runner.bytes_per_block) / 16
+        out = {"prefill_tok_s": prompt / t_prefill, "prefill_ms": 1e3 * t_prefill, "decode_tok_s": batch / t_decode,
+               "decode_ms_per_step": 1e3 * t_decode, "decode_weight_gb": weights / 1e9, "decode_kv_gb": kv / 1e9,
+               "decode_hbm_frac": (weights + kv) / t_decode / 1e9 / HBM_PEAK_GBS}
+        del runner
+        gc.collect()
+        torch.cuda.empty_cache()
+        return out
+
+    with tempfile.TemporaryDirectory(prefix="psamd_compare_") as tmp:
+        for name, size in sizes.items():
+            radivik, llama = radivik_pair(size, layers, vocab)
+            results[name] = {}
+            for design, cfg in (("radivik", radivik), ("llama", llama)):
+                if args.compare_only not in ("both", design):
+                    continue
+                folder = write_random_model(Path(tmp) / f"{name}-{design}", cfg, seed=0)
+                results[name][design] = measure(folder)
+            both = results[name]
+            if len(both) == 2:
+                both["radivik_over_llama"] = {k: both["radivik"][k] / both["llama"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+    print(json.dumps({"metric": "radivik_beside_llama_of_equal_size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
+                      "data": "synthetic: seeded uniform-random token ids, seeded random weights",
+                      "config": {"layers": layers, "vocab": vocab, "prompt_len": prompt, "decode_batch": batch,
+                                 "context": context, "steps": args.steps, "warmup": args.warmup},
+                      "sizes": results}), flush=True)
+    return 0
+
+
 def prefill_flops(cfg: dict, layers: int, tokens: int) -> float:
     h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     hq, hkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -92,10 +206,17 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
+    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"], default=None,
+                    help="instead of the benchmark: Radivik layers of this size beside Llama layers of equal size "
+                         "(prefill of --prompt-len tokens, decoding at --batch in --context; --layers, default 4)")
+    ap.add_argument("--compare-only", choices=["both", "radivik", "llama"], default="both")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.compare is not None:
+        return compare_designs(args)
 
     import numpy as np
     import torch

@@ -62,6 +62,16 @@ int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, c
                            int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
                            float up_shift);
 
+// The same for bfloat16 with the pairs sorted by expert and every expert's pairs run through its
+// matrices in tiles on the matrix cores. ints: scratch of pairs + 3 * psamd_moe_grouped_max_tiles(pairs,
+// experts) integers (pairs = tokens * top). K and F multiples of 8.
+int psamd_moe_grouped_tile_rows(int64_t pairs, int experts);
+int psamd_moe_grouped_max_tiles(int64_t pairs, int experts);
+int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
+                              const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
+                              int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
+                              float up_shift);
+
 // out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,
                  int64_t M, int N, int K);

@@ -1,7 +1,12 @@
-// Mixture-of-experts feed-forward: the router, and the experts one (token, choice) pair at a
-// time. The pair form reads an expert's matrices once per pair, which is what a decode step
-// needs (a handful of tokens, each with its own experts) and what the 32-bit path uses at every
-// size; it is templated on the element type (bfloat16 or float) and sums in float.
+// Mixture-of-experts feed-forward: the router, and the experts in two forms.
+//
+// * Pair by pair: one (token, choice) pair per workgroup row, the expert's matrices read once per
+//   pair. It is the form of the 32-bit path at every size (templated on the element type, sums in
+//   float, in an order that does not depend on the step) and of bfloat16 steps of one or two tokens.
+// * Grouped (bfloat16): the step's pairs are sorted by expert, and every expert's pairs go through
+//   its matrices in tiles of 16 or 64 pairs on the matrix cores (v_mfma_f32_16x16x32_bf16), so an
+//   expert is read once per tile of pairs instead of once per pair: a decode batch reads each
+//   expert it uses once, a prompt's portion runs as grouped products.
 //
 // Router: score = sigmoid(x . w_r[e]) in float; the `top` largest are taken, the lower index
 // among equals. Expert: with h = weight * x, g = min(gate h, limit), u = clamp(up h, -limit, limit),
@@ -14,6 +19,9 @@
 #include "common.h"
 
 namespace psamd {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 // Dot product of a row of n elements with a float vector in LDS, dealt out over the 64 lanes;
 // every lane returns the whole sum. bfloat16 rows whose length is a multiple of 8 are read in
@@ -147,6 +155,169 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(
   }
 }
 
+
+// ------------------------------------------------------------------ experts, grouped by expert
+
+// One workgroup sorts the step's pairs by expert and lists the tiles of `tile_rows` pairs the
+// products run over. ints: sorted[pairs] (pair indices, expert by expert), then per tile slot
+// tile_expert, tile_first (index into sorted), tile_count; slots past the last tile hold -1.
+// The order of an expert's pairs among themselves is whatever the atomics gave: every pair's
+// result is computed from its own row alone, so it does not matter which rows share a tile.
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restrict__ chosen, int pairs, int experts,
+                                                         int tile_rows, int max_tiles, int32_t* __restrict__ sorted,
+                                                         int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_first,
+                                                         int32_t* __restrict__ tile_count) {
+  extern __shared__ int32_t group_smem[];      // count[experts], start[experts], cursor[experts]
+  int32_t* count = group_smem;
+  int32_t* start = group_smem + experts;
+  int32_t* cursor = group_smem + 2 * experts;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = cursor[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[min(max(chosen[p], 0), experts - 1)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < experts; ++e) {
+      start[e] = at;
+      for (int r0 = 0; r0 < count[e] && nt < max_tiles; r0 += tile_rows, ++nt) {
+        tile_expert[nt] = e;
+        tile_first[nt] = at + r0;
+        tile_count[nt] = min(tile_rows, count[e] - r0);
+      }
+      at += count[e];
+    }
+    for (; nt < max_tiles; ++nt) tile_expert[nt] = -1;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = min(max(chosen[p], 0), experts - 1);
+    sorted[start[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+constexpr int kGroupBK = 128;                  // k per staging round
+constexpr int kGroupLD = kGroupBK + 8;         // LDS row stride of the staged pairs, in elements
+
+// One workgroup (4 waves) per (64 output columns, tile of MT * 16 pairs of one expert). The
+// pairs' input rows are staged in LDS 128 k at a time (gathered through `sorted`; GATED: the
+// token's row times the pair's weight, rounded to bfloat16 as the product's operand); every
+// wave streams its 16 rows of the expert's matrix from memory (GATED: 16 gate rows and the 16 up
+// rows that belong to them) and multiplies them with all MT tiles of pairs.
+//   GATED: out_act[pair][n] = act(gate, up) in bfloat16, N = F columns, w = [E][2N][K].
+//   else:  out_f32[(pair % top) * tokens + pair / top][n] = sum, N = hidden columns, w = [E][N][K],
+//          rows of `a` are indexed by pair.
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void moe_grouped_kernel(
+    const bf16_t* __restrict__ a, const float* __restrict__ pair_weight, const bf16_t* __restrict__ w,
+    const int32_t* __restrict__ sorted, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_first,
+    const int32_t* __restrict__ tile_count, bf16_t* __restrict__ out_act, float* __restrict__ out_f32, int64_t tokens,
+    int K, int N, int top, float gate_alpha, float limit, float up_shift) {
+  constexpr int ROWS = MT * 16;
+  __shared__ __align__(16) bf16_t as[ROWS * kGroupLD];
+  __shared__ int32_t pair_s[ROWS];
+  const int slot = blockIdx.y;
+  const int e = tile_expert[slot];
+  if (e < 0) return;                            // uniform for the workgroup
+  const int first = tile_first[slot], count = tile_count[slot];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = static_cast<int>(blockIdx.x) * 64 + wave * 16;
+  if (threadIdx.x < ROWS) pair_s[threadIdx.x] = threadIdx.x < count ? sorted[first + threadIdx.x] : -1;
+  const int nrow = min(n0 + r, N - 1);
+  const bf16_t* wg = w + (static_cast<int64_t>(e) * (GATED ? 2 : 1) * N + nrow) * K + 8 * g;
+  const bf16_t* wu = wg + static_cast<int64_t>(N) * K;     // GATED only
+  f32x4 acc_g[MT], acc_u[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc_g[mt] = acc_u[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += kGroupBK) {
+    if (k0 > 0) __syncthreads();                // the previous round's rows have been read
+    for (int idx = threadIdx.x; idx < ROWS * (kGroupBK / 8); idx += 256) {
+      const int row = idx / (kGroupBK / 8), c = idx - row * (kGroupBK / 8);
+      const int k = k0 + 8 * c;
+      const int pair = pair_s[row];
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (pair >= 0 && k < K) {
+        const int64_t src = GATED ? pair / top : pair;
+        v = *reinterpret_cast<const uint4*>(a + src * K + k);
+        if (GATED) {
+          const float s = pair_weight[pair];
+          uint32_t* u = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float lo = s * __uint_as_float(u[i] << 16), hi = s * __uint_as_float(u[i] & 0xffff0000u);
+            u[i] = static_cast<uint32_t>(float_to_bf16(lo)) | (static_cast<uint32_t>(float_to_bf16(hi)) << 16);
+          }
+        }
+      }
+      *reinterpret_cast<uint4*>(as + row * kGroupLD + 8 * c) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kGroupBK / 32; ++kk) {
+      const int k = k0 + kk * 32;
+      if (k >= K) break;                        // uniform
+      const bool in = k + 8 * g < K;            // K is a multiple of 8: a piece is inside or outside as a whole
+      bf16x8 wa, wb;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) wa[i] = wb[i] = static_cast<__bf16>(0.f);
+      if (in) {
+        wa = *reinterpret_cast<const bf16x8*>(wg + k);
+        if (GATED) wb = *reinterpret_cast<const bf16x8*>(wu + k);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(as + (mt * 16 + r) * kGroupLD + kk * 32 + 8 * g);
+        acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, b, acc_g[mt], 0, 0, 0);
+        if (GATED) acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, b, acc_u[mt], 0, 0, 0);
+      }
+    }
+  }
+  // Lane (r, g) holds, for the pair in row mt * 16 + r, the four columns n0 + 4 g .. + 3.
+  const int nc = n0 + 4 * g;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int pair = pair_s[mt * 16 + r];
+    if (pair < 0) continue;
+    if (GATED) {
+      bf16_t* o = out_act + static_cast<int64_t>(pair) * N + nc;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (nc + v >= N) break;
+        const float gg = fminf(acc_g[mt][v], limit);
+        const float uu = fminf(fmaxf(acc_u[mt][v], -limit), limit);
+        o[v] = float_to_bf16(gg / (1.f + __expf(-gate_alpha * gg)) * (uu + up_shift));
+      }
+    } else {
+      float* o = out_f32 + (static_cast<int64_t>(pair % top) * tokens + pair / top) * N + nc;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (nc + v >= N) break;
+        o[v] = acc_g[mt][v];
+      }
+    }
+  }
+}
+
+template <int MT>
+static int launch_grouped(hipStream_t s, const void* x, const float* weight, const void* w_gate_up, const void* w_down,
+                          void* act, float* out, const int32_t* ints, int max_tiles, int64_t tokens, int K, int F, int top,
+                          float gate_alpha, float limit, float up_shift) {
+  const int64_t pairs = tokens * top;
+  const int32_t* sorted = ints;
+  const int32_t* t_e = ints + pairs;
+  const int32_t* t_f = t_e + max_tiles;
+  const int32_t* t_c = t_f + max_tiles;
+  moe_grouped_kernel<MT, true><<<dim3(static_cast<unsigned>(ceil_div(F, 64)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
+      static_cast<const bf16_t*>(x), weight, static_cast<const bf16_t*>(w_gate_up), sorted, t_e, t_f, t_c,
+      static_cast<bf16_t*>(act), nullptr, tokens, K, F, top, gate_alpha, limit, up_shift);
+  if (check_launch("psamd_moe_experts_grouped (gate/up)")) return 1;
+  moe_grouped_kernel<MT, false><<<dim3(static_cast<unsigned>(ceil_div(K, 64)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
+      static_cast<const bf16_t*>(act), nullptr, static_cast<const bf16_t*>(w_down), sorted, t_e, t_f, t_c, nullptr, out,
+      tokens, F, K, top, 0.f, 0.f, 0.f);
+  return check_launch("psamd_moe_experts_grouped (down)");
+}
+
 template <typename A>
 static int launch_experts_rows(hipStream_t s, const void* x, const int32_t* chosen, const float* weight,
                                const void* w_gate_up, const void* w_down, void* act, float* out, int64_t tokens, int K,
@@ -206,6 +377,41 @@ int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, c
     return launch_experts_rows<float>(s, x, chosen, weight, w_gate_up, w_down, act, out, tokens, K, F, experts, top,
                                       gate_alpha, limit, up_shift);
   return fail("psamd_moe_experts_rows: dtype must be float32 or bfloat16");
+}
+
+// Pairs per tile of the grouped form for a step of this many pairs over this many experts: 64 when
+// the experts have that many pairs each on average, 16 below.
+int psamd_moe_grouped_tile_rows(int64_t pairs, int experts) { return pairs >= 32LL * experts ? 64 : 16; }
+
+// Tile slots the grouped form's grid has for such a step (every expert may end in a tile that is not full).
+int psamd_moe_grouped_max_tiles(int64_t pairs, int experts) {
+  const int rows = psamd_moe_grouped_tile_rows(pairs, experts);
+  return static_cast<int>(std::min<int64_t>(ceil_div(pairs, rows) + experts, pairs));
+}
+
+int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
+                              const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
+                              int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
+                              float up_shift) {
+  PSAMD_REQUIRE(tokens >= 0 && K > 0 && F > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
+  PSAMD_REQUIRE(K % 8 == 0 && F % 8 == 0, "K and F must be multiples of 8");
+  PSAMD_REQUIRE(experts <= 4096 && tokens * top <= (1 << 24), "too many experts or pairs");
+  PSAMD_REQUIRE(ints != nullptr, "the grouping needs its integer scratch");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t pairs = tokens * top;
+  const int rows = psamd_moe_grouped_tile_rows(pairs, experts);
+  const int max_tiles = psamd_moe_grouped_max_tiles(pairs, experts);
+  PSAMD_REQUIRE(max_tiles <= 65535, "too many tiles for one launch");
+  moe_group_kernel<<<dim3(1), dim3(1024), sizeof(int32_t) * 3 * experts, s>>>(
+      chosen, static_cast<int>(pairs), experts, rows, max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
+      ints + pairs + 2 * max_tiles);
+  if (check_launch("psamd_moe_experts_grouped (grouping)")) return 1;
+  if (rows == 64)
+    return launch_grouped<4>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
+                             up_shift);
+  return launch_grouped<1>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
+                           up_shift);
 }
 
 }  // extern "C"

@@ -73,6 +73,8 @@ _SIGNATURES = {
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
     "psamd_rope_norm_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp],
     "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_moe_grouped_max_tiles": [_i64, _i32],
+    "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
     "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
 }
 
@@ -82,6 +84,7 @@ class HipOps:
     SKINNY_MAX_ROWS = 64
     FUSED_SWIGLU_MAX_ROWS = 32      # above it (to SKINNY_MAX_ROWS) gate/up goes to the library, where there is one
     LIBRARY_ADD_MIN_ROWS = 1024     # from here on a product that feeds the residual stream adds into it in the library
+    MOE_PAIRWISE_MAX_TOKENS = 2     # up to here a bfloat16 step's experts run pair by pair; above, grouped by expert
     name = "hip"
 
     def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
@@ -499,6 +502,15 @@ class HipOps:
                    "moe_experts: the router's outputs")
         self._need(act.shape == (t * top, f) and act.dtype == x.dtype and act.is_contiguous(), "moe_experts: act scratch")
         self._need(out.shape == (top, t, k) and out.dtype == torch.float32 and out.is_contiguous(), "moe_experts: output slices")
+        if x.dtype == torch.bfloat16 and t > self.MOE_PAIRWISE_MAX_TOKENS and k % 8 == 0 and f % 8 == 0:
+            # Sorted by expert and run in tiles on the matrix cores: an expert is read once per tile of pairs.
+            tiles = int(self.lib.psamd_moe_grouped_max_tiles(t * top, e))
+            ints = self.ws.get("moe.group", (t * top + 3 * tiles,), torch.int32)
+            self._ok(self.lib.psamd_moe_experts_grouped(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
+                                                        w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(),
+                                                        out.data_ptr(), ints.data_ptr(), t, k, f, e, top, float(gate_alpha),
+                                                        float(limit), float(up_shift)))
+            return
         self._ok(self.lib.psamd_moe_experts_rows(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
                                                  w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(), out.data_ptr(),
                                                  _code(x.dtype), t, k, f, e, top, float(gate_alpha), float(limit),

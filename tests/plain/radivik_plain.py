@@ -97,10 +97,15 @@ def sigmoid(z: np.ndarray) -> np.ndarray:
     return 1.0 / (1.0 + np.exp(-z))
 
 
-def expert(h: np.ndarray, gate: np.ndarray, up: np.ndarray, down: np.ndarray, limit: float) -> np.ndarray:
-    g = np.minimum(h @ gate.T, limit)
-    u = np.clip(h @ up.T, -limit, limit)
-    return (g * sigmoid(1.702 * g) * (u + 1.0)) @ down.T
+def _same(x: np.ndarray) -> np.ndarray:
+    return x
+
+
+def expert(h: np.ndarray, gate: np.ndarray, up: np.ndarray, down: np.ndarray, limit: float, r: Any = _same) -> np.ndarray:
+    """``r`` rounds what a 16-bit engine would keep in 16 bits (a product's output, an activation)."""
+    g = np.minimum(r(h @ gate.T), limit)
+    u = np.clip(r(h @ up.T), -limit, limit)
+    return r(g * sigmoid(1.702 * g) * (u + 1.0)) @ down.T
 
 
 def route(h: np.ndarray, router: np.ndarray, top: int) -> tuple[np.ndarray, np.ndarray]:
@@ -111,12 +116,12 @@ def route(h: np.ndarray, router: np.ndarray, top: int) -> tuple[np.ndarray, np.n
 
 
 def mixture(h: np.ndarray, router: np.ndarray, experts: list[tuple[np.ndarray, np.ndarray, np.ndarray]], top: int,
-            limit: float) -> np.ndarray:
+            limit: float, r: Any = _same) -> np.ndarray:
     chosen, score = route(h, router, top)
     out = np.zeros((h.shape[0], experts[0][2].shape[0]), dtype=h.dtype)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t], score[t]):
-            out[t] += expert(w * h[t], *experts[int(e)], limit)
+            out[t] += expert(r(w * h[t]), *experts[int(e)], limit, r)
     return out
 
 
@@ -124,8 +129,13 @@ def mixture(h: np.ndarray, router: np.ndarray, experts: list[tuple[np.ndarray, n
 
 
 class PlainRadivik:
-    def __init__(self, model_dir: str | Path, dtype: Any = np.float64) -> None:
+    def __init__(self, model_dir: str | Path, dtype: Any = np.float64, bf16: bool = False) -> None:
+        """``bf16``: the yardstick for a 16-bit engine. The outputs of products and the activations
+        between them are rounded to bfloat16; what the design computes in 32-bit (angles, unit
+        norms, scores and softmax, router, the sum and the norm behind it) is float32."""
         model_dir = Path(model_dir)
+        self.r = (lambda x: round_bf16(x).astype(np.float32)) if bf16 else _same
+        dtype = np.float32 if bf16 else dtype
         self.cfg = json.loads((model_dir / "config.json").read_text())
         self.w = {k: (v.astype(dtype) if v.dtype.kind == "f" else v)
                   for k, v in read_safetensors(model_dir / "model.safetensors").items()}
@@ -137,28 +147,31 @@ class PlainRadivik:
         m = self.cfg["layers"][i]["mixer"]
         n, p = x.shape[0], f"l{i}.mix."
         freq, gain = yarn_frequencies(int(m["rot"]["dims"]), float(m["rot"]["base"]), m["rot"].get("scaling"))
-        k = (x @ self.w[p + "k"].T).reshape(n, int(m["kv_heads"]), int(m["dim"]))
-        v = (x @ self.w[p + "v"].T).reshape(n, int(m["kv_heads"]), int(m["vdim"]))
-        return unit_rms(rotate(k, pos, freq, gain), self.eps), v
+        r = self.r
+        k = r(x @ self.w[p + "k"].T).reshape(n, int(m["kv_heads"]), int(m["dim"]))
+        v = r(x @ self.w[p + "v"].T).reshape(n, int(m["kv_heads"]), int(m["vdim"]))
+        return r(unit_rms(rotate(k, pos, freq, gain), self.eps).astype(self.dtype)), v
 
     def mixer(self, i: int, x: np.ndarray, pos: np.ndarray, kept: dict[int, Any]) -> np.ndarray:
         m = self.cfg["layers"][i]["mixer"]
         n, p = x.shape[0], f"l{i}.mix."
         freq, gain = yarn_frequencies(int(m["rot"]["dims"]), float(m["rot"]["base"]), m["rot"].get("scaling"))
-        q = (x @ self.w[p + "q"].T).reshape(n, int(m["heads"]), int(m["dim"]))
-        q = unit_rms(rotate(q, pos, freq, gain), self.eps)
+        r = self.r
+        x = r(x)
+        q = r(x @ self.w[p + "q"].T).reshape(n, int(m["heads"]), int(m["dim"]))
+        q = r(unit_rms(rotate(q, pos, freq, gain), self.eps).astype(self.dtype))
         if m.get("kv_from") is not None:
             k, v = kept[int(m["kv_from"])]
         else:
             k, v = kept[i] = self.keys_values(i, x, pos)
-        return attend(q, k, v, float(m["scale"])).reshape(n, -1) @ self.w[p + "o"].T
+        return r(r(attend(q, k, v, float(m["scale"])).reshape(n, -1)) @ self.w[p + "o"].T)
 
     def feed_forward(self, i: int, x: np.ndarray) -> np.ndarray:
         f = self.cfg["layers"][i]["mlp"]
         p = f"l{i}.mlp."
         experts = [(self.w[f"{p}e{e}.gate"], self.w[f"{p}e{e}.up"], self.w[f"{p}e{e}.down"])
                    for e in range(int(f["router"]["experts"]))]
-        return mixture(x, self.w[p + "router"], experts, int(f["router"]["top"]), float(f["expert"]["limit"]))
+        return mixture(self.r(x), self.w[p + "router"], experts, int(f["router"]["top"]), float(f["expert"]["limit"]), self.r)
 
     def hidden(self, tokens: Any, every_layer: bool = False) -> Any:
         ids = np.asarray(tokens, dtype=np.int64)
@@ -175,7 +188,7 @@ class PlainRadivik:
         return np.stack(trail) if every_layer else x
 
     def logits(self, tokens: Any) -> np.ndarray:
-        return rms_norm(self.hidden(tokens), self.w["final.norm"], self.eps) @ self.w["head"].T
+        return self.r(rms_norm(self.hidden(tokens), self.w["final.norm"], self.eps)) @ self.w["head"].T
 
     def greedy(self, prompt: Any, steps: int) -> list[int]:
         ids = [int(t) for t in prompt]
