@@ -141,6 +141,14 @@ def compare_designs(args) -> int:
             decode()
         t_decode = timed(decode, args.steps)
         weights = runner.model.step_weight_bytes()
+        # A mixture of experts reads every expert some token of the batch has chosen: with uniform choices,
+        # experts x (1 - (1 - top / experts)^batch) of them, where one token reads top.
+        for blk in runner.model.blocks:
+            ff = getattr(blk, "feed_forward", None)
+            if ff is not None and hasattr(ff, "num_experts"):
+                per_expert = (ff.w_gate_up.numel() + ff.w_down.numel()) // ff.num_experts * ff.w_down.element_size()
+                used = ff.num_experts * (1.0 - (1.0 - ff.top_k / ff.num_experts) ** batch)
+                weights += (used - ff.top_k) * per_expert
         kv = batch * (fill + args.steps / 2) * sum(runner.bytes_per_block) / 16
         out = {"prefill_tok_s": prompt / t_prefill, "prefill_ms": 1e3 * t_prefill, "decode_tok_s": batch / t_decode,
                "decode_ms_per_step": 1e3 * t_decode, "decode_weight_gb": weights / 1e9, "decode_kv_gb": kv / 1e9,

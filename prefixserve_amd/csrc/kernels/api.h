@@ -54,6 +54,9 @@ int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t to
 // first), weight[t, :] = those scores.
 int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_router, int32_t* chosen, float* weight,
                     int64_t tokens, int K, int experts, int top);
+// The same choice from logits that a product has written (float [tokens, experts]).
+int psamd_moe_topk(void* stream, const float* logits, int32_t* chosen, float* weight, int64_t tokens, int experts,
+                   int top);
 // Experts, one (token, choice) pair at a time: h = weight[t, j] * x[t]; g = min(gate h, limit), u =
 // clamp(up h, -limit, limit); act[t * top + j] = g * sigmoid(gate_alpha * g) * (u + up_shift);
 // out[j][t] = down act (float). w_gate_up is [E, 2F, K] (gate rows, then up rows), w_down [E, K, F].

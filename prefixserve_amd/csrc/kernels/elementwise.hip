@@ -426,6 +426,73 @@ __global__ __launch_bounds__(kThreads) void scaled_add_rmsnorm_kernel(
   }
 }
 
+// The same for rows that are a multiple of 4 wide, up to 4 * kThreads * kIter: every thread owns
+// runs of 4 consecutive elements (16-byte accesses of the stream and of float slices), and up to
+// four slices are asked for together and added in ascending order.
+template <typename A, typename DT, int kThreads, int kIter>
+__global__ __launch_bounds__(kThreads) void scaled_add_rmsnorm_vec4_kernel(
+    float* __restrict__ residual, float alpha, const DT* __restrict__ delta, int n_partials, int64_t partial_stride,
+    const void* __restrict__ weight, int weight_dtype, float eps, A* __restrict__ out, int hidden) {
+  __shared__ float scratch[kThreads / kWave];
+  float* r = residual + static_cast<int64_t>(blockIdx.x) * hidden;
+  const DT* d0 = delta != nullptr ? delta + static_cast<int64_t>(blockIdx.x) * hidden : nullptr;
+  A* o = out != nullptr ? out + static_cast<int64_t>(blockIdx.x) * hidden : nullptr;
+  const int np = delta != nullptr ? n_partials : 0;
+  const int chunks = hidden >> 2;
+  float4 v[kIter];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < kIter; ++j) {
+    const int cidx = static_cast<int>(threadIdx.x) + j * kThreads;
+    const int e = min(cidx, chunks - 1) << 2;
+    float4 x = *reinterpret_cast<const float4*>(r + e);
+    x.x *= alpha; x.y *= alpha; x.z *= alpha; x.w *= alpha;
+    if (sizeof(DT) == 2) {
+      if (np > 0) {
+        const uint2 q = *reinterpret_cast<const uint2*>(d0 + e);
+        x.x += __uint_as_float(q.x << 16); x.y += __uint_as_float(q.x & 0xffff0000u);
+        x.z += __uint_as_float(q.y << 16); x.w += __uint_as_float(q.y & 0xffff0000u);
+      }
+    } else {
+      for (int p = 0; p < np; p += 4) {
+        float4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          t[u] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(d0) + min(p + u, np - 1) * partial_stride + e);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (p + u < np) { x.x += t[u].x; x.y += t[u].y; x.z += t[u].z; x.w += t[u].w; }
+        }
+      }
+    }
+    v[j] = x;
+    if (cidx < chunks) ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+  }
+  ss = block_sum(ss, scratch, kThreads / kWave);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+  for (int j = 0; j < kIter; ++j) {
+    const int cidx = static_cast<int>(threadIdx.x) + j * kThreads;
+    if (cidx >= chunks) continue;
+    const int e = cidx << 2;
+    float4 y;
+    y.x = load_as_float(weight, weight_dtype, e) * (v[j].x * inv);
+    y.y = load_as_float(weight, weight_dtype, e + 1) * (v[j].y * inv);
+    y.z = load_as_float(weight, weight_dtype, e + 2) * (v[j].z * inv);
+    y.w = load_as_float(weight, weight_dtype, e + 3) * (v[j].w * inv);
+    *reinterpret_cast<float4*>(r + e) = y;
+    if (o != nullptr) {
+      if (sizeof(A) == 2) {
+        ushort4 pk;
+        pk.x = float_to_bf16(y.x); pk.y = float_to_bf16(y.y); pk.z = float_to_bf16(y.z); pk.w = float_to_bf16(y.w);
+        *reinterpret_cast<ushort4*>(reinterpret_cast<bf16_t*>(o) + e) = pk;
+      } else {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(o) + e) = y;
+      }
+    }
+  }
+}
+
 // out[i] = A(in[i]): the float32 stream in the activation type.
 template <typename A>
 __global__ void to_activation_kernel(const float* __restrict__ in, A* __restrict__ out, int64_t n) {
@@ -637,7 +704,28 @@ int psamd_scaled_add_rmsnorm(void* stream, float* residual, float alpha, const v
       residual, alpha, static_cast<const D_*>(delta), n_partials, partial_stride, weight, weight_dtype, eps, \
       static_cast<A_*>(out), hidden)
   const bool delta_f32 = delta == nullptr || delta_dtype == kF32;
-  if (out != nullptr && act_dtype == kBF16) {
+  const bool out_bf16 = out != nullptr && act_dtype == kBF16;
+  if (hidden % 4 == 0 && hidden <= 4 * kThreads * 8 && (partial_stride % 4 == 0 || n_partials <= 1)) {
+#define PSAMD_POSTNORM4(A_, D_, IT_)                                                                        \
+  scaled_add_rmsnorm_vec4_kernel<A_, D_, kThreads, IT_><<<grid, block, 0, s>>>(                             \
+      residual, alpha, static_cast<const D_*>(delta), n_partials, partial_stride, weight, weight_dtype, eps, \
+      static_cast<A_*>(out), hidden)
+#define PSAMD_POSTNORM4_IT(A_, D_)                                                 \
+  do {                                                                             \
+    if (hidden <= 4 * kThreads * 2) PSAMD_POSTNORM4(A_, D_, 2);                    \
+    else if (hidden <= 4 * kThreads * 4) PSAMD_POSTNORM4(A_, D_, 4);               \
+    else PSAMD_POSTNORM4(A_, D_, 8);                                               \
+  } while (0)
+    if (out_bf16) {
+      if (delta_f32) PSAMD_POSTNORM4_IT(bf16_t, float); else PSAMD_POSTNORM4_IT(bf16_t, bf16_t);
+    } else {
+      if (delta_f32) PSAMD_POSTNORM4_IT(float, float); else PSAMD_POSTNORM4_IT(float, bf16_t);
+    }
+#undef PSAMD_POSTNORM4_IT
+#undef PSAMD_POSTNORM4
+    return check_launch("psamd_scaled_add_rmsnorm");
+  }
+  if (out_bf16) {
     if (delta_f32) PSAMD_POSTNORM(bf16_t, float); else PSAMD_POSTNORM(bf16_t, bf16_t);
   } else {
     if (delta_f32) PSAMD_POSTNORM(float, float); else PSAMD_POSTNORM(float, bf16_t);

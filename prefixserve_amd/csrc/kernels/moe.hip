@@ -41,6 +41,20 @@ __device__ __forceinline__ float wave_dot(const W* __restrict__ row, const float
         acc = fmaf(__uint_as_float(w4[i] & 0xffff0000u), xp[2 * i + 1], acc);
       }
     }
+  } else if (sizeof(W) == 4 && (n & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int chunks = n >> 2;
+    float acc2 = 0.f;
+    for (int c = lane; c < chunks; c += 2 * kWave) {
+      const int c2 = c + kWave;
+      const float4 q = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(row) + 4 * c);
+      const float4 q2 = c2 < chunks ? *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(row) + 4 * c2)
+                                    : float4{0.f, 0.f, 0.f, 0.f};
+      const float* xp = xs + 4 * c;
+      const float* xp2 = xs + 4 * min(c2, chunks - 1);
+      acc = fmaf(q.x, xp[0], acc); acc = fmaf(q.y, xp[1], acc); acc = fmaf(q.z, xp[2], acc); acc = fmaf(q.w, xp[3], acc);
+      acc2 = fmaf(q2.x, xp2[0], acc2); acc2 = fmaf(q2.y, xp2[1], acc2); acc2 = fmaf(q2.z, xp2[2], acc2); acc2 = fmaf(q2.w, xp2[3], acc2);
+    }
+    acc += acc2;
   } else {
     for (int i = lane; i < n; i += kWave) acc = fmaf(to_float<W>(row[i]), xs[i], acc);
   }
@@ -75,6 +89,47 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const A* __restrict__ x,
     for (int e = lane; e < experts; e += kWave) {
       const float s = score[e];
       if (s > best) {                                    // ascending e: the first of equals stays
+        best = s;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, kWave);
+      const int oa = __shfl_xor(at, o, kWave);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    if (lane == 0) {
+      chosen[t * top + j] = at;
+      weight[t * top + j] = best;
+      score[at] = -2.f;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+}
+
+// The same choice from logits a product has already written: z[t, :] float -> sigmoid, the `top`
+// largest. One wave per token, four tokens per block.
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen,
+                                                       float* __restrict__ weight, int64_t tokens, int experts, int top) {
+  extern __shared__ __align__(16) float topk_smem[];     // score[4][experts]
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  if (t >= tokens) return;
+  float* score = topk_smem + wave * experts;
+  for (int e = lane; e < experts; e += kWave) score[e] = 1.f / (1.f + expf(-z[t * experts + e]));
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  for (int j = 0; j < top; ++j) {
+    float best = -1.f;
+    int at = 0x7fffffff;
+    for (int e = lane; e < experts; e += kWave) {
+      const float s = score[e];
+      if (s > best) {
         best = s;
         at = e;
       }
@@ -195,25 +250,30 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
   }
 }
 
-constexpr int kGroupBK = 128;                  // k per staging round
+constexpr int kGroupBK = 64;                   // k per staging round
 constexpr int kGroupLD = kGroupBK + 8;         // LDS row stride of the staged pairs, in elements
 
-// One workgroup (4 waves) per (64 output columns, tile of MT * 16 pairs of one expert). The
-// pairs' input rows are staged in LDS 128 k at a time (gathered through `sorted`; GATED: the
+// One workgroup (4 waves) per (64 * RT output columns, tile of MT * 16 pairs of one expert). The
+// pairs' input rows pass through LDS 64 k at a time (gathered through `sorted`; GATED: the
 // token's row times the pair's weight, rounded to bfloat16 as the product's operand); every
-// wave streams its 16 rows of the expert's matrix from memory (GATED: 16 gate rows and the 16 up
-// rows that belong to them) and multiplies them with all MT tiles of pairs.
+// wave streams its 16 * RT rows of the expert's matrix from memory (GATED: gate rows and the up
+// rows that belong to them) and multiplies them with all MT tiles of pairs. The next round's
+// rows of both operands are asked for before the current round is multiplied (registers, then
+// the other of two LDS buffers), so one barrier per round is all the waves wait for.
 //   GATED: out_act[pair][n] = act(gate, up) in bfloat16, N = F columns, w = [E][2N][K].
 //   else:  out_f32[(pair % top) * tokens + pair / top][n] = sum, N = hidden columns, w = [E][N][K],
 //          rows of `a` are indexed by pair.
-template <int MT, bool GATED>
+template <int MT, int RT, bool GATED>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const bf16_t* __restrict__ a, const float* __restrict__ pair_weight, const bf16_t* __restrict__ w,
     const int32_t* __restrict__ sorted, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_first,
     const int32_t* __restrict__ tile_count, bf16_t* __restrict__ out_act, float* __restrict__ out_f32, int64_t tokens,
     int K, int N, int top, float gate_alpha, float limit, float up_shift) {
   constexpr int ROWS = MT * 16;
-  __shared__ __align__(16) bf16_t as[ROWS * kGroupLD];
+  constexpr int PIECES = ROWS * (kGroupBK / 8);              // 16-byte pieces of a round's pairs
+  constexpr int PPT = (PIECES + 255) / 256;                  // pieces per thread
+  constexpr int KK = kGroupBK / 32;
+  __shared__ __align__(16) bf16_t as[2][ROWS * kGroupLD];
   __shared__ int32_t pair_s[ROWS];
   const int slot = blockIdx.y;
   const int e = tile_expert[slot];
@@ -221,85 +281,142 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   const int first = tile_first[slot], count = tile_count[slot];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = static_cast<int>(blockIdx.x) * 64 + wave * 16;
+  const int n0 = (static_cast<int>(blockIdx.x) * 4 + wave) * 16 * RT;     // this wave's first column
   if (threadIdx.x < ROWS) pair_s[threadIdx.x] = threadIdx.x < count ? sorted[first + threadIdx.x] : -1;
-  const int nrow = min(n0 + r, N - 1);
-  const bf16_t* wg = w + (static_cast<int64_t>(e) * (GATED ? 2 : 1) * N + nrow) * K + 8 * g;
-  const bf16_t* wu = wg + static_cast<int64_t>(N) * K;     // GATED only
-  f32x4 acc_g[MT], acc_u[MT];
+  const bf16_t* wg[RT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc_g[mt] = acc_u[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt) {
+    const int nrow = min(n0 + rt * 16 + r, N - 1);
+    wg[rt] = w + (static_cast<int64_t>(e) * (GATED ? 2 : 1) * N + nrow) * K + 8 * g;
+  }
+  const int64_t up_off = static_cast<int64_t>(N) * K;                      // GATED: from a gate row to its up row
+  f32x4 acc_g[RT][MT], acc_u[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc_g[rt][mt] = acc_u[rt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   __syncthreads();
-  for (int k0 = 0; k0 < K; k0 += kGroupBK) {
-    if (k0 > 0) __syncthreads();                // the previous round's rows have been read
-    for (int idx = threadIdx.x; idx < ROWS * (kGroupBK / 8); idx += 256) {
-      const int row = idx / (kGroupBK / 8), c = idx - row * (kGroupBK / 8);
-      const int k = k0 + 8 * c;
-      const int pair = pair_s[row];
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (pair >= 0 && k < K) {
-        const int64_t src = GATED ? pair / top : pair;
-        v = *reinterpret_cast<const uint4*>(a + src * K + k);
-        if (GATED) {
-          const float s = pair_weight[pair];
-          uint32_t* u = reinterpret_cast<uint32_t*>(&v);
+
+  // This thread's pieces of a round: which pair's row, where from, its weight.
+  const bf16_t* src[PPT];
+  float scale[PPT];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float lo = s * __uint_as_float(u[i] << 16), hi = s * __uint_as_float(u[i] & 0xffff0000u);
-            u[i] = static_cast<uint32_t>(float_to_bf16(lo)) | (static_cast<uint32_t>(float_to_bf16(hi)) << 16);
-          }
+  for (int p = 0; p < PPT; ++p) {
+    const int idx = static_cast<int>(threadIdx.x) + p * 256;
+    const int row = min(idx, PIECES - 1) / (kGroupBK / 8), c = min(idx, PIECES - 1) % (kGroupBK / 8);
+    const int pair = pair_s[row];
+    src[p] = (pair >= 0 && idx < PIECES) ? a + static_cast<int64_t>(GATED ? pair / top : pair) * K + 8 * c : nullptr;
+    scale[p] = (GATED && pair >= 0) ? pair_weight[pair] : 1.f;
+  }
+  uint4 areg[PPT];
+  bf16x8 wa[KK][RT], wb[KK][RT];
+  auto ask = [&](int k0) {                       // the round's rows of both operands, into registers
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) {
+      const int c8 = 8 * ((static_cast<int>(threadIdx.x) + p * 256) % (kGroupBK / 8));
+      areg[p] = (src[p] != nullptr && k0 + c8 < K) ? *reinterpret_cast<const uint4*>(src[p] + k0) : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int k = k0 + kk * 32;
+      const bool in = k + 8 * g < K;            // K is a multiple of 8: a piece is inside or outside as a whole
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wa[kk][rt][i] = wb[kk][rt][i] = static_cast<__bf16>(0.f);
+        if (in) {
+          wa[kk][rt] = *reinterpret_cast<const bf16x8*>(wg[rt] + k);
+          if (GATED) wb[kk][rt] = *reinterpret_cast<const bf16x8*>(wg[rt] + up_off + k);
         }
       }
-      *reinterpret_cast<uint4*>(as + row * kGroupLD + 8 * c) = v;
     }
-    __syncthreads();
+  };
+  auto stage = [&](int buf) {                    // the pairs' pieces from registers into LDS, weighted
 #pragma unroll
-    for (int kk = 0; kk < kGroupBK / 32; ++kk) {
-      const int k = k0 + kk * 32;
-      if (k >= K) break;                        // uniform
-      const bool in = k + 8 * g < K;            // K is a multiple of 8: a piece is inside or outside as a whole
-      bf16x8 wa, wb;
+    for (int p = 0; p < PPT; ++p) {
+      const int idx = static_cast<int>(threadIdx.x) + p * 256;
+      if (idx >= PIECES) continue;
+      uint4 v = areg[p];
+      if (GATED) {
+        uint32_t* u = reinterpret_cast<uint32_t*>(&v);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) wa[i] = wb[i] = static_cast<__bf16>(0.f);
-      if (in) {
-        wa = *reinterpret_cast<const bf16x8*>(wg + k);
-        if (GATED) wb = *reinterpret_cast<const bf16x8*>(wu + k);
+        for (int i = 0; i < 4; ++i) {
+          const float lo = scale[p] * __uint_as_float(u[i] << 16), hi = scale[p] * __uint_as_float(u[i] & 0xffff0000u);
+          u[i] = static_cast<uint32_t>(float_to_bf16(lo)) | (static_cast<uint32_t>(float_to_bf16(hi)) << 16);
+        }
       }
+      *reinterpret_cast<uint4*>(as[buf] + (idx / (kGroupBK / 8)) * kGroupLD + 8 * (idx % (kGroupBK / 8))) = v;
+    }
+  };
+  ask(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += kGroupBK, buf ^= 1) {
+    bf16x8 ca[KK][RT], cb[KK][RT];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        ca[kk][rt] = wa[kk][rt];
+        cb[kk][rt] = wb[kk][rt];
+      }
+    const bool more = k0 + kGroupBK < K;
+    if (more) ask(k0 + kGroupBK);               // in flight while this round is multiplied
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 b = *reinterpret_cast<const bf16x8*>(as + (mt * 16 + r) * kGroupLD + kk * 32 + 8 * g);
-        acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, b, acc_g[mt], 0, 0, 0);
-        if (GATED) acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, b, acc_u[mt], 0, 0, 0);
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(as[buf] + (mt * 16 + r) * kGroupLD + kk * 32 + 8 * g);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          acc_g[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca[kk][rt], b, acc_g[rt][mt], 0, 0, 0);
+          if (GATED) acc_u[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb[kk][rt], b, acc_u[rt][mt], 0, 0, 0);
+        }
       }
     }
+    if (more) stage(buf ^ 1);                   // nobody reads that buffer: all passed the last barrier after reading it
+    __syncthreads();
   }
-  // Lane (r, g) holds, for the pair in row mt * 16 + r, the four columns n0 + 4 g .. + 3.
-  const int nc = n0 + 4 * g;
+  // Lane (r, g) holds, for the pair in row mt * 16 + r, the four columns n0 + rt * 16 + 4 g .. + 3.
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int pair = pair_s[mt * 16 + r];
     if (pair < 0) continue;
-    if (GATED) {
-      bf16_t* o = out_act + static_cast<int64_t>(pair) * N + nc;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        if (nc + v >= N) break;
-        const float gg = fminf(acc_g[mt][v], limit);
-        const float uu = fminf(fmaxf(acc_u[mt][v], -limit), limit);
-        o[v] = float_to_bf16(gg / (1.f + __expf(-gate_alpha * gg)) * (uu + up_shift));
-      }
-    } else {
-      float* o = out_f32 + (static_cast<int64_t>(pair % top) * tokens + pair / top) * N + nc;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int nc = n0 + rt * 16 + 4 * g;
+      if (GATED) {
+        bf16_t* o = out_act + static_cast<int64_t>(pair) * N + nc;
+        bf16_t res[4];
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        if (nc + v >= N) break;
-        o[v] = acc_g[mt][v];
+        for (int v = 0; v < 4; ++v) {
+          const float gg = fminf(acc_g[rt][mt][v], limit);
+          const float uu = fminf(fmaxf(acc_u[rt][mt][v], -limit), limit);
+          res[v] = float_to_bf16(gg / (1.f + __expf(-gate_alpha * gg)) * (uu + up_shift));
+        }
+        if (nc + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<ushort4*>(o) = ushort4{res[0], res[1], res[2], res[3]};
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nc + v < N) o[v] = res[v];
+        }
+      } else {
+        float* o = out_f32 + (static_cast<int64_t>(pair % top) * tokens + pair / top) * N + nc;
+        if (nc + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<float4*>(o) = float4{acc_g[rt][mt][0], acc_g[rt][mt][1], acc_g[rt][mt][2], acc_g[rt][mt][3]};
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nc + v < N) o[v] = acc_g[rt][mt][v];
+        }
       }
     }
   }
 }
 
-template <int MT>
+template <int MT, int RT>
 static int launch_grouped(hipStream_t s, const void* x, const float* weight, const void* w_gate_up, const void* w_down,
                           void* act, float* out, const int32_t* ints, int max_tiles, int64_t tokens, int K, int F, int top,
                           float gate_alpha, float limit, float up_shift) {
@@ -308,11 +425,11 @@ static int launch_grouped(hipStream_t s, const void* x, const float* weight, con
   const int32_t* t_e = ints + pairs;
   const int32_t* t_f = t_e + max_tiles;
   const int32_t* t_c = t_f + max_tiles;
-  moe_grouped_kernel<MT, true><<<dim3(static_cast<unsigned>(ceil_div(F, 64)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
+  moe_grouped_kernel<MT, RT, true><<<dim3(static_cast<unsigned>(ceil_div(F, 64 * RT)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
       static_cast<const bf16_t*>(x), weight, static_cast<const bf16_t*>(w_gate_up), sorted, t_e, t_f, t_c,
       static_cast<bf16_t*>(act), nullptr, tokens, K, F, top, gate_alpha, limit, up_shift);
   if (check_launch("psamd_moe_experts_grouped (gate/up)")) return 1;
-  moe_grouped_kernel<MT, false><<<dim3(static_cast<unsigned>(ceil_div(K, 64)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
+  moe_grouped_kernel<MT, RT, false><<<dim3(static_cast<unsigned>(ceil_div(K, 64 * RT)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
       static_cast<const bf16_t*>(act), nullptr, static_cast<const bf16_t*>(w_down), sorted, t_e, t_f, t_c, nullptr, out,
       tokens, F, K, top, 0.f, 0.f, 0.f);
   return check_launch("psamd_moe_experts_grouped (down)");
@@ -361,6 +478,17 @@ int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_rou
   return check_launch("psamd_moe_route");
 }
 
+int psamd_moe_topk(void* stream, const float* logits, int32_t* chosen, float* weight, int64_t tokens, int experts,
+                   int top) {
+  PSAMD_REQUIRE(tokens >= 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
+  PSAMD_REQUIRE(sizeof(float) * 4 * static_cast<size_t>(experts) <= 64 * 1024, "scores do not fit in LDS");
+  PSAMD_REQUIRE(ceil_div(tokens, 4) <= 2147483647LL, "too many tokens for one launch");
+  if (tokens == 0) return 0;
+  moe_topk_kernel<<<dim3(static_cast<unsigned>(ceil_div(tokens, 4))), dim3(256), sizeof(float) * 4 * experts,
+                    static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, tokens, experts, top);
+  return check_launch("psamd_moe_topk");
+}
+
 int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, const float* weight,
                            const void* w_gate_up, const void* w_down, void* act, float* out, int dtype,
                            int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
@@ -379,9 +507,11 @@ int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, c
   return fail("psamd_moe_experts_rows: dtype must be float32 or bfloat16");
 }
 
-// Pairs per tile of the grouped form for a step of this many pairs over this many experts: 64 when
-// the experts have that many pairs each on average, 16 below.
-int psamd_moe_grouped_tile_rows(int64_t pairs, int experts) { return pairs >= 32LL * experts ? 64 : 16; }
+// Pairs per tile of the grouped form for a step of this many pairs over this many experts: 128 or 64
+// when the experts have about that many pairs each on average, 16 below.
+int psamd_moe_grouped_tile_rows(int64_t pairs, int experts) {
+  return pairs >= 96LL * experts ? 128 : (pairs >= 32LL * experts ? 64 : 16);
+}
 
 // Tile slots the grouped form's grid has for such a step (every expert may end in a tile that is not full).
 int psamd_moe_grouped_max_tiles(int64_t pairs, int experts) {
@@ -407,11 +537,14 @@ int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen
       chosen, static_cast<int>(pairs), experts, rows, max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
       ints + pairs + 2 * max_tiles);
   if (check_launch("psamd_moe_experts_grouped (grouping)")) return 1;
+  if (rows == 128)
+    return launch_grouped<8, 2>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha,
+                                limit, up_shift);
   if (rows == 64)
-    return launch_grouped<4>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
-                             up_shift);
-  return launch_grouped<1>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
-                           up_shift);
+    return launch_grouped<4, 2>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha,
+                                limit, up_shift);
+  return launch_grouped<1, 1>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
+                              up_shift);
 }
 
 }  // extern "C"

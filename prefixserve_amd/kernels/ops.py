@@ -73,6 +73,7 @@ _SIGNATURES = {
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
     "psamd_rope_norm_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp],
     "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_moe_grouped_max_tiles": [_i64, _i32],
     "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
     "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
@@ -84,6 +85,7 @@ class HipOps:
     SKINNY_MAX_ROWS = 64
     FUSED_SWIGLU_MAX_ROWS = 32      # above it (to SKINNY_MAX_ROWS) gate/up goes to the library, where there is one
     LIBRARY_ADD_MIN_ROWS = 1024     # from here on a product that feeds the residual stream adds into it in the library
+    MOE_ROUTE_FUSED_MAX_TOKENS = 0   # up to here one kernel computes router logits and choice; above, product + choice
     MOE_PAIRWISE_MAX_TOKENS = 2     # up to here a bfloat16 step's experts run pair by pair; above, grouped by expert
     name = "hip"
 
@@ -473,11 +475,25 @@ class HipOps:
 
     # ------------------------------------------------------------------ experts
 
-    def moe_route(self, x, w_router, chosen, weight) -> None:
+    def moe_route(self, x, w_router, chosen, weight, w_router_act=None) -> None:
         """chosen[t, :], weight[t, :] = the experts with the largest sigmoid(x[t] . w_router[e]) and
-        those scores, largest first, the lower index among equals; scores in 32-bit."""
+        those scores, largest first, the lower index among equals; scores in 32-bit. With the router
+        also given in the activation dtype (``w_router_act``), a step of more than
+        ``MOE_ROUTE_FUSED_MAX_TOKENS`` tokens takes its logits from the product kernels (float32 sums of
+        exact products, float32 out) and the choice from a kernel of its own: the fused kernel reads
+        the whole router once per token with one workgroup (8 tokens of a 32 x 2,048 router: 94 us
+        against 5 + 4 for product and choice), so the bound is 0 and it serves callers without that copy."""
         t, k = x.shape
         e, top = w_router.shape[0], chosen.shape[1]
+        if (w_router_act is not None and t > self.MOE_ROUTE_FUSED_MAX_TOKENS and w_router_act.dtype == x.dtype
+                and w_router_act.shape == w_router.shape and 1 <= top <= e):
+            self._need(chosen.dtype == torch.int32 and weight.dtype == torch.float32 and chosen.shape == (t, top)
+                       and weight.shape == (t, top) and chosen.is_contiguous() and weight.is_contiguous(),
+                       "moe_route: outputs must be int32 and float32 [T, top]")
+            logits = self.ws.get("moe.logits", (t, e), torch.float32)
+            self.linear(x, w_router_act, logits)
+            self._ok(self.lib.psamd_moe_topk(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(), t, e, top))
+            return
         self._need(x.is_contiguous() and w_router.dtype == torch.float32 and w_router.is_contiguous()
                    and w_router.shape[1] == k, "moe_route: x [T, K], router float32 [E, K]")
         self._need(chosen.dtype == torch.int32 and weight.dtype == torch.float32 and chosen.shape == (t, top)

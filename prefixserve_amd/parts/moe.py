@@ -55,6 +55,9 @@ class RoutedExperts(FeedForward):
         n, e_n = self.names, self.num_experts
         # The router stays 32-bit whatever the activation dtype.
         self.w_router = tensors[n["router"]].to(device=rt.device, dtype=torch.float32).contiguous()
+        # ... and also stands in the activation dtype for steps whose logits a product kernel computes
+        # (bfloat16 x bfloat16 products are exact in float32, where they are summed).
+        self.w_router_act = self.w_router if rt.dtype == torch.float32 else rt.ops.prepare_matrix(tensors[n["router"]], rt)
         # Per expert the rows of gate, then of up: [E, 2F, H]; and down [E, H, F].
         gate_up = torch.stack([torch.cat([tensors[n["gate"].format(e=e)], tensors[n["up"].format(e=e)]], dim=0)
                                for e in range(e_n)])
@@ -71,7 +74,7 @@ class RoutedExperts(FeedForward):
         t, k = x.shape[0], self.top_k
         chosen = ws.get("moe.chosen", (t, k), torch.int32)
         weight = ws.get("moe.weight", (t, k), torch.float32)
-        ops.moe_route(x, self.w_router, chosen, weight)
+        ops.moe_route(x, self.w_router, chosen, weight, self.w_router_act)
         act = ws.get("moe.act", (t * k, self.intermediate_size), rt.dtype)
         out = ws.get("moe.out", (k, t, self.hidden_size), torch.float32)
         ops.moe_experts(x, chosen, weight, self.w_gate_up, self.w_down, act, out, self.gate_alpha, self.limit, self.up_shift)

@@ -114,7 +114,7 @@ class EmulatedOps:
             kv[:, 0].view(kv.shape[0], hkv, PAGE, d)[page, :, off, :] = heads[:, hq:]
             kv[:, 1].view(kv.shape[0], hkv, d, PAGE)[page, :, :, off] = qkv[:, (hq + hkv) * d:].view(t, hkv, d)
 
-    def moe_route(self, x, w_router, chosen, weight) -> None:
+    def moe_route(self, x, w_router, chosen, weight, w_router_act=None) -> None:
         s = torch.sigmoid(x.float() @ w_router.float().T)
         order = torch.argsort(-s, dim=-1, stable=True)[:, : chosen.shape[1]]
         chosen.copy_(order.to(torch.int32))

@@ -53,12 +53,14 @@ def rel(got, want):
 # ------------------------------------------------------------------ kernels
 
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hidden,form", [(96, "none"), (192, "plain"), (1000, "slices"), (4104, "slices"), (4104, "plain")])
+@pytest.mark.parametrize("hidden,form", [(96, "none"), (192, "plain"), (1000, "slices"), (4104, "slices"), (4104, "plain"),
+                                         (998, "slices"), (999, "plain"), (8192, "slices"), (8200, "slices"), (2048, "five")])
 def test_norm_behind_the_sum(ops, act, hidden, form):
     t, eps, alpha = 5, 1e-5, 1.75
     res = rnd(t, hidden, seed=1)
     w = (1 + 0.1 * rnd(hidden, seed=3)).to(torch.bfloat16)
-    delta = {"none": None, "plain": rnd(t, hidden, dtype=act, seed=2), "slices": rnd(3, t, hidden, seed=2)}[form]
+    delta = {"none": None, "plain": rnd(t, hidden, dtype=act, seed=2), "slices": rnd(3, t, hidden, seed=2),
+             "five": rnd(5, t, hidden, seed=2)}[form]
     x = alpha * res.double()
     if delta is not None:
         x = x + (delta.double().sum(0) if delta.dim() == 3 else delta.double())
@@ -117,15 +119,15 @@ def test_rope_norm_kv_append(ops, act, hq, hkv, d, norm_dim):
 
 
 @pytest.mark.parametrize("act", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("t,k,e,top", [(1, 96, 5, 2), (9, 64, 4, 4), (70, 128, 9, 1), (3, 200, 130, 8)])
+@pytest.mark.parametrize("t,k,e,top", [(1, 96, 5, 2), (9, 64, 4, 4), (70, 128, 9, 1), (3, 200, 130, 8), (333, 256, 40, 6), (17, 100, 7, 3)])
 def test_router_picks_the_largest_scores(ops, act, t, k, e, top):
     x = rnd(t, k, dtype=act, seed=7)
-    w = rnd(e, k, seed=8, scale=0.3)
+    w = rnd(e, k, seed=8, scale=0.3).to(torch.bfloat16).float()       # a router as checkpoints store it
     if e >= 4:
         w[3] = w[1]                                                    # equal scores: the lower index wins
     chosen = torch.empty(t, top, dtype=torch.int32, device=DEV)
     weight = torch.empty(t, top, device=DEV)
-    ops.moe_route(x, w, chosen, weight)
+    ops.moe_route(x, w, chosen, weight, w.to(act))                     # more than 16 tokens: product kernel + choice
     want_e, want_s = plain.route(x.double().cpu().numpy(), w.double().cpu().numpy(), top)
     s = plain.sigmoid(x.double().cpu().numpy() @ w.double().cpu().numpy().T)
     got_e = chosen.cpu().numpy()
@@ -146,8 +148,9 @@ def test_experts_weight_their_input_and_clamp(ops, act, t, k, f, e, top, limit):
     x = rnd(t, k, dtype=act, seed=9)
     gate_up = rnd(e, 2 * f, k, dtype=act, seed=10, scale=0.15)
     down = rnd(e, k, f, dtype=act, seed=11, scale=0.15)
-    chosen = torch.stack([torch.randperm(e)[:top] for _ in range(t)]).to(torch.int32).to(DEV)
-    weight = torch.rand(t, top).to(DEV)
+    gen = torch.Generator().manual_seed(12)
+    chosen = torch.stack([torch.randperm(e, generator=gen)[:top] for _ in range(t)]).to(torch.int32).to(DEV)
+    weight = (0.4 + 0.6 * torch.rand(t, top, generator=gen)).to(DEV)
     act_buf = torch.empty(t * top, f, dtype=act, device=DEV)
     out = torch.full((top, t, k), 3.0, device=DEV)
     ops.moe_experts(x, chosen, weight, gate_up, down, act_buf, out, 1.702, limit, 1.0)
@@ -160,7 +163,7 @@ def test_experts_weight_their_input_and_clamp(ops, act, t, k, f, e, top, limit):
             h = float(weight[i, j]) * xs[i]
             want[j, i] = plain.expert(h, gu[ex, :f], gu[ex, f:], dn[ex], limit)
             clamped += int((np.abs(gu[ex, f:] @ h) > limit).sum() + ((gu[ex, :f] @ h) > limit).sum())
-    assert clamped > 0 or limit > 5                                    # the clamps are at work in this test
+    assert clamped > 0 or limit > 5 or t < 4                           # the clamps are at work in this test
     assert rel(out, want) < (1e-5 if act == torch.float32 else 2e-2)
 
 
