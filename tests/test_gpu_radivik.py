@@ -375,3 +375,89 @@ def test_the_replay_program_on_a_radivik_folder(folders, tmp_path):
             got = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(exp), -1)
             for row, (i, p) in zip(got, exp):
                 assert rel(row, truth[i][p]) < tol, (dtype, s["step"], i, p)
+
+
+def _random_radivik(rng) -> dict:
+    """A configuration drawn at random: sizes that are no multiples of 8 or 16, head sizes in either
+    order, rotations from none of the head to all of it, layers that read earlier layers, layers
+    without a feed-forward, one to all experts per token."""
+    width = int(rng.choice([40, 72, 100, 136, 192]))
+    mixers = []
+    for _ in range(int(rng.integers(1, 3))):
+        kv_heads = int(rng.choice([1, 2, 3]))
+        dim = int(rng.choice([8, 20, 32, 48, 72]))
+        dims = int(rng.choice([0, 2, dim // 2 // 2 * 2, dim // 2 * 2]))
+        scaling = None if rng.random() < 0.3 else {"factor": float(rng.choice([1.0, 2.0, 8.0, 40.0])), "original": int(rng.choice([16, 64, 512])),
+                                                    "fast": float(rng.choice([4.0, 32.0])), "slow": float(rng.choice([0.25, 1.0, 2.0]))}
+        rot = {"base": float(rng.choice([10.0, 10000.0, 1e6])), "dims": dims}
+        if scaling is not None:
+            rot["scaling"] = scaling
+        mixers.append({"heads": kv_heads * int(rng.choice([1, 2, 4])), "kv_heads": kv_heads, "dim": dim,
+                       "vdim": int(rng.choice([8, 12, 32, 40, 80])), "scale": float(rng.choice([0.1, 0.3, 0.7])), "rot": rot})
+    layers, owners = [], {}
+    for i in range(int(rng.integers(2, 6))):
+        which = int(rng.integers(0, len(mixers)))
+        m = dict(mixers[which])
+        if which in owners and rng.random() < 0.5:
+            m["kv_from"] = int(rng.choice(owners[which]))
+        else:
+            owners.setdefault(which, []).append(i)
+        experts = int(rng.integers(1, 13))
+        mlp = None if rng.random() < 0.2 else {"kind": "moe", "router": {"experts": experts, "top": int(rng.integers(1, min(experts, 4) + 1))},
+                                               "expert": {"ff": int(rng.choice([8, 20, 36, 64])), "limit": float(rng.choice([0.3, 1.0, 4.0]))}}
+        layers.append({"type": "attention", "mixer": m, "mlp": mlp})
+    return {"architecture": "Radivik", "vocab": int(rng.choice([50, 131, 300])), "width": width,
+            "norm": {"eps": float(rng.choice([1e-6, 1e-5, 1e-3]))}, "postln_alpha": float(rng.choice([0.5, 1.0, 2.0, 4.0])), "layers": layers}
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations_in_both_dtypes(seed, tmp_path):
+    rng = np.random.default_rng(4000 + seed)
+    cfg = _random_radivik(rng)
+    folder = write_radivik(tmp_path, "", seed=seed, config=cfg)
+    model = plain.PlainRadivik(folder)
+    reqs = [rng.integers(0, cfg["vocab"], n).tolist() for n in (75, 40, 97, 18, 66)]
+    truth = [model.logits(t) for t in reqs]
+    mean_bar, row_bar = bf16_bars(folder, truth, reqs)
+    for dtype in ("float32", "bfloat16"):
+        tol = 2e-5 if dtype == "float32" else max(2.0 * row_bar, 0.05)
+        runner = runner_for(folder, dtype, 32)
+        errors = []
+        for build in (traces.decode_tail, traces.portions):
+            steps, expect = build(reqs)
+            traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, tol, errors)
+        steps, expect, peak = traces.mixed(reqs, seed=seed)
+        small = runner_for(folder, dtype, peak // 16)
+        for t in small.pools.tensors:
+            t.fill_(1e30)
+        traces.compare(TraceReplayer(small).run_step, steps, expect, truth, tol, errors)
+        shape = [(l["mixer"]["heads"], l["mixer"]["kv_heads"], l["mixer"]["dim"], l["mixer"]["vdim"], l["mixer"]["rot"]["dims"],
+                  l["mixer"].get("kv_from"), None if l["mlp"] is None else (l["mlp"]["router"]["experts"], l["mlp"]["router"]["top"],
+                                                                         l["mlp"]["expert"]["ff"])) for l in cfg["layers"]]
+        print(seed, dtype, cfg["width"], shape, f"worst {max(errors):.2e} mean {np.mean(errors):.2e} (plain bf16 {mean_bar:.2e}, row {row_bar:.2e})")
+        if dtype == "bfloat16":
+            assert np.mean(errors) <= 1.5 * mean_bar + 2e-3           # an expert score that nearly ties may fall the other way
+
+
+def test_the_command_line_on_a_radivik_folder(tmp_path):
+    """``random-model`` writes a Radivik folder from its config.json, ``generate`` runs it: the same
+    commands as for any other architecture, chosen by the file."""
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(RADIVIK["R"]))
+    proc = subprocess.run([sys.executable, "-m", "prefixserve_amd.cli", "random-model", "--config", str(cfg),
+                           "--out", str(tmp_path / "m"), "--seed", "9"], capture_output=True, text=True, cwd=ROOT)
+    assert proc.returncode == 0 and (tmp_path / "m" / "model.safetensors").exists(), proc.stderr
+    # the default spread of 0.02 leaves near-ties; the comparison is on a folder with the tests' spread
+    folder = write_radivik(tmp_path / "w", "R", seed=9)
+    prompt = [5, 17, 3, 190, 41, 7, 7, 19, 0, 64, 11]
+    want = plain.PlainRadivik(folder).greedy(prompt, 6)
+    for model in (tmp_path / "m", folder):
+        proc = subprocess.run(
+            [sys.executable, "-m", "prefixserve_amd.cli", "generate", "--model", str(model), "--dtype", "float32",
+             "--max-seq-len", "128", "--num-blocks", "16", "--max-running-requests", "2", "--chunked-prefill-size", "5",
+             "--max-tokens", "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt))],
+            capture_output=True, text=True, cwd=ROOT, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        out = json.loads(proc.stdout.strip().splitlines()[-1])
+        assert len(out["outputs"][0]["tokens"]) == 6 and out["outputs"][0]["finish_reason"] == "length"
+    assert out["outputs"][0]["tokens"] == want
