@@ -73,7 +73,11 @@ int psamd_moe_grouped_max_tiles(int64_t pairs, int experts);
 int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
                               const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
                               int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                              float up_shift);
+                              float up_shift, int grouped_already);
+// psamd_moe_topk and the sorting of the pairs into `ints` in one workgroup, for up to 64 tokens;
+// psamd_moe_experts_grouped is then called with grouped_already = 1 and the same `ints`.
+int psamd_moe_topk_group(void* stream, const float* logits, int32_t* chosen, float* weight, int32_t* ints, int64_t tokens,
+                         int experts, int top);
 
 // out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,

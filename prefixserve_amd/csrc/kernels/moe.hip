@@ -218,14 +218,12 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(
 // tile_expert, tile_first (index into sorted), tile_count; slots past the last tile hold -1.
 // The order of an expert's pairs among themselves is whatever the atomics gave: every pair's
 // result is computed from its own row alone, so it does not matter which rows share a tile.
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restrict__ chosen, int pairs, int experts,
-                                                         int tile_rows, int max_tiles, int32_t* __restrict__ sorted,
-                                                         int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_first,
-                                                         int32_t* __restrict__ tile_count) {
-  extern __shared__ int32_t group_smem[];      // count[experts], start[experts], cursor[experts]
-  int32_t* count = group_smem;
-  int32_t* start = group_smem + experts;
-  int32_t* cursor = group_smem + 2 * experts;
+// `count`, `start`, `tstart`, `cursor` are LDS arrays of `experts` integers each.
+__device__ __forceinline__ void group_pairs(const int32_t* __restrict__ chosen, int pairs, int experts, int tile_rows,
+                                            int max_tiles, int32_t* __restrict__ sorted, int32_t* __restrict__ tile_expert,
+                                            int32_t* __restrict__ tile_first, int32_t* __restrict__ tile_count,
+                                            int32_t* count, int32_t* start, int32_t* tstart, int32_t* cursor,
+                                            int32_t* n_tiles) {
   for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = cursor[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[min(max(chosen[p], 0), experts - 1)], 1);
@@ -234,28 +232,93 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restri
     int at = 0, nt = 0;
     for (int e = 0; e < experts; ++e) {
       start[e] = at;
-      for (int r0 = 0; r0 < count[e] && nt < max_tiles; r0 += tile_rows, ++nt) {
-        tile_expert[nt] = e;
-        tile_first[nt] = at + r0;
-        tile_count[nt] = min(tile_rows, count[e] - r0);
-      }
+      tstart[e] = nt;
       at += count[e];
+      nt += (count[e] + tile_rows - 1) / tile_rows;
     }
-    for (; nt < max_tiles; ++nt) tile_expert[nt] = -1;
+    *n_tiles = min(nt, max_tiles);
   }
   __syncthreads();
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+    int nt = tstart[e];
+    for (int r0 = 0; r0 < count[e] && nt < max_tiles; r0 += tile_rows, ++nt) {
+      tile_expert[nt] = e;
+      tile_first[nt] = start[e] + r0;
+      tile_count[nt] = min(tile_rows, count[e] - r0);
+    }
+  }
+  for (int nt = *n_tiles + threadIdx.x; nt < max_tiles; nt += blockDim.x) tile_expert[nt] = -1;
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
     const int e = min(max(chosen[p], 0), experts - 1);
     sorted[start[e] + atomicAdd(&cursor[e], 1)] = p;
   }
 }
 
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* __restrict__ chosen, int pairs, int experts,
+                                                         int tile_rows, int max_tiles, int32_t* __restrict__ sorted,
+                                                         int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_first,
+                                                         int32_t* __restrict__ tile_count) {
+  extern __shared__ int32_t group_smem[];      // count, start, tstart, cursor [experts] each, n_tiles
+  group_pairs(chosen, pairs, experts, tile_rows, max_tiles, sorted, tile_expert, tile_first, tile_count, group_smem,
+              group_smem + experts, group_smem + 2 * experts, group_smem + 3 * experts, group_smem + 4 * experts);
+}
+
+// The choice from logits and the sorting in one workgroup of 16 waves, for steps of so few tokens
+// that one workgroup does the choice at once (a decode step): a wave per token, then the sorting above.
+__global__ __launch_bounds__(1024) void moe_topk_group_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen,
+                                                              float* __restrict__ weight, int tokens, int experts, int top,
+                                                              int tile_rows, int max_tiles, int32_t* __restrict__ sorted,
+                                                              int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_first,
+                                                              int32_t* __restrict__ tile_count) {
+  extern __shared__ int32_t group_smem[];      // as above, then score[16][experts]
+  float* score = reinterpret_cast<float*>(group_smem + 4 * experts + 1) + (threadIdx.x >> 6) * experts;
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int t = threadIdx.x >> 6; t < tokens; t += 16) {
+    for (int e = lane; e < experts; e += kWave) score[e] = 1.f / (1.f + expf(-z[static_cast<int64_t>(t) * experts + e]));
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int j = 0; j < top; ++j) {
+      float best = -1.f;
+      int at = 0x7fffffff;
+      for (int e = lane; e < experts; e += kWave) {
+        const float s = score[e];
+        if (s > best) {
+          best = s;
+          at = e;
+        }
+      }
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, kWave);
+        const int oa = __shfl_xor(at, o, kWave);
+        if (ob > best || (ob == best && oa < at)) {
+          best = ob;
+          at = oa;
+        }
+      }
+      if (lane == 0) {
+        chosen[t * top + j] = at;
+        weight[t * top + j] = best;
+        score[at] = -2.f;
+      }
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+    }
+  }
+  __threadfence_block();
+  __syncthreads();                             // the workgroup's own writes of `chosen` are read below
+  group_pairs(chosen, tokens * top, experts, tile_rows, max_tiles, sorted, tile_expert, tile_first, tile_count, group_smem,
+              group_smem + experts, group_smem + 2 * experts, group_smem + 3 * experts, group_smem + 4 * experts);
+}
+
 constexpr int kGroupBK = 64;                   // k per staging round
 constexpr int kGroupLD = kGroupBK + 8;         // LDS row stride of the staged pairs, in elements
 
 // One workgroup (4 waves) per (64 * RT output columns, tile of MT * 16 pairs of one expert). The
-// pairs' input rows pass through LDS 64 k at a time (gathered through `sorted`; GATED: the
-// token's row times the pair's weight, rounded to bfloat16 as the product's operand); every
+// pairs' input rows pass through LDS 64 k at a time (gathered through `sorted`). GATED: the
+// pair's weight on the expert's input is applied to the float32 sums, gate (w x) = w (gate x),
+// before the clamps: the same number without a rounding of w x, and no arithmetic while staging
+// (scaling and rounding the rows there cost as many vector cycles as the matrix instructions). Every
 // wave streams its 16 * RT rows of the expert's matrix from memory (GATED: gate rows and the up
 // rows that belong to them) and multiplies them with all MT tiles of pairs. The next round's
 // rows of both operands are asked for before the current round is multiplied (registers, then
@@ -299,14 +362,12 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 
   // This thread's pieces of a round: which pair's row, where from, its weight.
   const bf16_t* src[PPT];
-  float scale[PPT];
 #pragma unroll
   for (int p = 0; p < PPT; ++p) {
     const int idx = static_cast<int>(threadIdx.x) + p * 256;
     const int row = min(idx, PIECES - 1) / (kGroupBK / 8), c = min(idx, PIECES - 1) % (kGroupBK / 8);
     const int pair = pair_s[row];
     src[p] = (pair >= 0 && idx < PIECES) ? a + static_cast<int64_t>(GATED ? pair / top : pair) * K + 8 * c : nullptr;
-    scale[p] = (GATED && pair >= 0) ? pair_weight[pair] : 1.f;
   }
   uint4 areg[PPT];
   bf16x8 wa[KK][RT], wb[KK][RT];
@@ -331,21 +392,12 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       }
     }
   };
-  auto stage = [&](int buf) {                    // the pairs' pieces from registers into LDS, weighted
+  auto stage = [&](int buf) {                    // the pairs' pieces from registers into LDS
 #pragma unroll
     for (int p = 0; p < PPT; ++p) {
       const int idx = static_cast<int>(threadIdx.x) + p * 256;
       if (idx >= PIECES) continue;
-      uint4 v = areg[p];
-      if (GATED) {
-        uint32_t* u = reinterpret_cast<uint32_t*>(&v);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float lo = scale[p] * __uint_as_float(u[i] << 16), hi = scale[p] * __uint_as_float(u[i] & 0xffff0000u);
-          u[i] = static_cast<uint32_t>(float_to_bf16(lo)) | (static_cast<uint32_t>(float_to_bf16(hi)) << 16);
-        }
-      }
-      *reinterpret_cast<uint4*>(as[buf] + (idx / (kGroupBK / 8)) * kGroupLD + 8 * (idx % (kGroupBK / 8))) = v;
+      *reinterpret_cast<uint4*>(as[buf] + (idx / (kGroupBK / 8)) * kGroupLD + 8 * (idx % (kGroupBK / 8))) = areg[p];
     }
   };
   ask(0);
@@ -383,6 +435,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   for (int mt = 0; mt < MT; ++mt) {
     const int pair = pair_s[mt * 16 + r];
     if (pair < 0) continue;
+    const float pw = GATED ? pair_weight[pair] : 1.f;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const int nc = n0 + rt * 16 + 4 * g;
@@ -391,8 +444,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
         bf16_t res[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          const float gg = fminf(acc_g[rt][mt][v], limit);
-          const float uu = fminf(fmaxf(acc_u[rt][mt][v], -limit), limit);
+          const float gg = fminf(pw * acc_g[rt][mt][v], limit);
+          const float uu = fminf(fmaxf(pw * acc_u[rt][mt][v], -limit), limit);
           res[v] = float_to_bf16(gg / (1.f + __expf(-gate_alpha * gg)) * (uu + up_shift));
         }
         if (nc + 3 < N && (N & 3) == 0) {
@@ -457,6 +510,9 @@ using namespace psamd;
 
 extern "C" {
 
+int psamd_moe_grouped_tile_rows(int64_t pairs, int experts);
+int psamd_moe_grouped_max_tiles(int64_t pairs, int experts);
+
 int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_router, int32_t* chosen, float* weight,
                     int64_t tokens, int K, int experts, int top) {
   PSAMD_REQUIRE(tokens >= 0 && K > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
@@ -487,6 +543,20 @@ int psamd_moe_topk(void* stream, const float* logits, int32_t* chosen, float* we
   moe_topk_kernel<<<dim3(static_cast<unsigned>(ceil_div(tokens, 4))), dim3(256), sizeof(float) * 4 * experts,
                     static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, tokens, experts, top);
   return check_launch("psamd_moe_topk");
+}
+
+int psamd_moe_topk_group(void* stream, const float* logits, int32_t* chosen, float* weight, int32_t* ints, int64_t tokens,
+                         int experts, int top) {
+  PSAMD_REQUIRE(tokens >= 1 && tokens <= 64 && experts > 0 && experts <= 1024 && top >= 1 && top <= experts, "bad sizes");
+  PSAMD_REQUIRE(ints != nullptr, "the grouping needs its integer scratch");
+  const int64_t pairs = tokens * top;
+  const int rows = psamd_moe_grouped_tile_rows(pairs, experts);
+  const int max_tiles = psamd_moe_grouped_max_tiles(pairs, experts);
+  moe_topk_group_kernel<<<dim3(1), dim3(1024), sizeof(int32_t) * (4 * experts + 1) + sizeof(float) * 16 * experts,
+                          static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, static_cast<int>(tokens), experts, top, rows,
+                                                              max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
+                                                              ints + pairs + 2 * max_tiles);
+  return check_launch("psamd_moe_topk_group");
 }
 
 int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, const float* weight,
@@ -522,7 +592,7 @@ int psamd_moe_grouped_max_tiles(int64_t pairs, int experts) {
 int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
                               const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
                               int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                              float up_shift) {
+                              float up_shift, int grouped_already) {
   PSAMD_REQUIRE(tokens >= 0 && K > 0 && F > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(K % 8 == 0 && F % 8 == 0, "K and F must be multiples of 8");
   PSAMD_REQUIRE(experts <= 4096 && tokens * top <= (1 << 24), "too many experts or pairs");
@@ -533,10 +603,12 @@ int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen
   const int rows = psamd_moe_grouped_tile_rows(pairs, experts);
   const int max_tiles = psamd_moe_grouped_max_tiles(pairs, experts);
   PSAMD_REQUIRE(max_tiles <= 65535, "too many tiles for one launch");
-  moe_group_kernel<<<dim3(1), dim3(1024), sizeof(int32_t) * 3 * experts, s>>>(
-      chosen, static_cast<int>(pairs), experts, rows, max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
-      ints + pairs + 2 * max_tiles);
-  if (check_launch("psamd_moe_experts_grouped (grouping)")) return 1;
+  if (grouped_already == 0) {
+    moe_group_kernel<<<dim3(1), dim3(1024), sizeof(int32_t) * (4 * experts + 1), s>>>(
+        chosen, static_cast<int>(pairs), experts, rows, max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
+        ints + pairs + 2 * max_tiles);
+    if (check_launch("psamd_moe_experts_grouped (grouping)")) return 1;
+  }
   if (rows == 128)
     return launch_grouped<8, 2>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha,
                                 limit, up_shift);

@@ -75,7 +75,8 @@ _SIGNATURES = {
     "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
     "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_moe_grouped_max_tiles": [_i64, _i32],
-    "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
+    "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32],
+    "psamd_moe_topk_group": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
 }
 
@@ -492,8 +493,17 @@ class HipOps:
                        "moe_route: outputs must be int32 and float32 [T, top]")
             logits = self.ws.get("moe.logits", (t, e), torch.float32)
             self.linear(x, w_router_act, logits)
+            self._grouped_for = None
+            if self._groups_pairs(x.dtype, t, k) and t <= 64 and e <= 1024:
+                # A small step: the workgroup that chooses also sorts the pairs for the experts' kernels.
+                ints = self._group_ints(t, top, e)
+                self._ok(self.lib.psamd_moe_topk_group(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
+                                                       ints.data_ptr(), t, e, top))
+                self._grouped_for = (chosen.data_ptr(), t, top, e)
+                return
             self._ok(self.lib.psamd_moe_topk(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(), t, e, top))
             return
+        self._grouped_for = None
         self._need(x.is_contiguous() and w_router.dtype == torch.float32 and w_router.is_contiguous()
                    and w_router.shape[1] == k, "moe_route: x [T, K], router float32 [E, K]")
         self._need(chosen.dtype == torch.int32 and weight.dtype == torch.float32 and chosen.shape == (t, top)
@@ -501,6 +511,14 @@ class HipOps:
                    "moe_route: outputs must be int32 and float32 [T, top]")
         self._ok(self.lib.psamd_moe_route(self._stream(), x.data_ptr(), _code(x.dtype), w_router.data_ptr(),
                                           chosen.data_ptr(), weight.data_ptr(), t, k, e, top))
+
+    def _groups_pairs(self, dtype: torch.dtype, t: int, k: int) -> bool:
+        """Whether a step of ``t`` tokens of width ``k`` runs its experts grouped by expert."""
+        return dtype == torch.bfloat16 and t > self.MOE_PAIRWISE_MAX_TOKENS and k % 8 == 0
+
+    def _group_ints(self, t: int, top: int, e: int) -> torch.Tensor:
+        tiles = int(self.lib.psamd_moe_grouped_max_tiles(t * top, e))
+        return self.ws.get("moe.group", (t * top + 3 * tiles,), torch.int32)
 
     def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha: float, limit: float,
                     up_shift: float) -> None:
@@ -518,14 +536,15 @@ class HipOps:
                    "moe_experts: the router's outputs")
         self._need(act.shape == (t * top, f) and act.dtype == x.dtype and act.is_contiguous(), "moe_experts: act scratch")
         self._need(out.shape == (top, t, k) and out.dtype == torch.float32 and out.is_contiguous(), "moe_experts: output slices")
-        if x.dtype == torch.bfloat16 and t > self.MOE_PAIRWISE_MAX_TOKENS and k % 8 == 0 and f % 8 == 0:
+        if self._groups_pairs(x.dtype, t, k) and f % 8 == 0:
             # Sorted by expert and run in tiles on the matrix cores: an expert is read once per tile of pairs.
-            tiles = int(self.lib.psamd_moe_grouped_max_tiles(t * top, e))
-            ints = self.ws.get("moe.group", (t * top + 3 * tiles,), torch.int32)
+            ints = self._group_ints(t, top, e)
+            done = int(getattr(self, "_grouped_for", None) == (chosen.data_ptr(), t, top, e))   # the router's kernel sorted them
+            self._grouped_for = None
             self._ok(self.lib.psamd_moe_experts_grouped(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
                                                         w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(),
                                                         out.data_ptr(), ints.data_ptr(), t, k, f, e, top, float(gate_alpha),
-                                                        float(limit), float(up_shift)))
+                                                        float(limit), float(up_shift), done))
             return
         self._ok(self.lib.psamd_moe_experts_rows(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
                                                  w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(), out.data_ptr(),
