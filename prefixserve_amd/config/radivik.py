@@ -10,7 +10,7 @@ load and then compute something else.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Any, Mapping
 
 from .llama import UnsupportedModelError
@@ -113,6 +113,9 @@ class RadivikExperts:
 class RadivikLayer:
     mixer: RadivikAttention
     mlp: RadivikExperts | None
+    # A layer without a feed-forward has no second half; if its checkpoint nevertheless brings a
+    # second norm, that norm is applied to the stream alone: x <- norm2(alpha x).
+    lone_second_norm: bool = False
 
 
 @dataclass(frozen=True)
@@ -147,6 +150,12 @@ class RadivikConfig:
             if (a.kv_heads, a.dim, a.vdim) != (b.kv_heads, b.dim, b.vdim):
                 raise UnsupportedModelError(f"layers[{i}] reads layer {j}'s keys and values but has other sizes")
         return cls(int(raw["vocab"]), int(raw["width"]), float(raw["norm"]["eps"]), float(raw["postln_alpha"]), tuple(layers))
+
+    def fitted_to_checkpoint(self, names: frozenset[str]) -> "RadivikConfig":
+        """The configuration with what the checkpoint's tensor names decide."""
+        layers = tuple(replace(layer, lone_second_norm=layer.mlp is None and f"l{i}.norm2" in names)
+                       for i, layer in enumerate(self.layers))
+        return replace(self, layers=layers)
 
     def to_config_json(self) -> dict[str, Any]:
         return {

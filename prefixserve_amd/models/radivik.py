@@ -56,6 +56,8 @@ def build_radivik_spec(cfg: RadivikConfig) -> ModelSpec:
                 "limit": f.limit, "gate_alpha": GATE_ALPHA, "up_shift": UP_SHIFT,
             })
             ff_norm = PartSpec("rmsnorm", {"eps": cfg.norm_eps, "name": "norm2"})
+        elif layer.lone_second_norm:
+            ff_norm = PartSpec("rmsnorm", {"eps": cfg.norm_eps, "name": "norm2"})
         layers.append(LayerSpec(
             prefix=f"l{i}.", mixer=mixer, feed_forward=ff,
             mixer_norm=PartSpec("rmsnorm", {"eps": cfg.norm_eps, "name": "norm1"}), feed_forward_norm=ff_norm,

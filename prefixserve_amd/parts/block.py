@@ -53,7 +53,8 @@ class PostNormBlock:
     on the stream in front of each sum (1: the plain arrangement). Sum, statistics and the
     stream are float32; beside the stream the norm writes its copy in the activation dtype
     for the next sub-layer's products (``ctx.stream_copy``, so that the next block of this
-    kind does not convert again). ``feed_forward`` None: the second half does not exist."""
+    kind does not convert again). ``feed_forward`` None: the second half does not exist, unless a
+    second norm is given all the same, which is then applied to the stream alone, norm2(alpha x)."""
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm,
                  feed_forward_norm: Norm | None, alpha: float = 1.0) -> None:
@@ -63,7 +64,9 @@ class PostNormBlock:
 
     def parts(self) -> list[Part]:
         both = [self.mixer_norm, self.mixer]
-        return both + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
+        if self.feed_forward is not None:
+            return both + [self.feed_forward_norm, self.feed_forward]
+        return both + ([self.feed_forward_norm] if self.feed_forward_norm is not None else [])
 
     def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
                 state: torch.Tensor | None, writes_cache: bool) -> None:
@@ -82,6 +85,8 @@ class PostNormBlock:
         x = self.mixer_norm.norm_of_sum(residual, mixed, self.alpha, "block.x")
         if self.feed_forward is not None:
             x = self.feed_forward_norm.norm_of_sum(residual, self.feed_forward.forward(x, ctx), self.alpha, "block.x")
+        elif self.feed_forward_norm is not None:
+            x = self.feed_forward_norm.norm_of_sum(residual, None, self.alpha, "block.x")
         ctx.stream_copy = x
         ctx.residual = kept
         return None

@@ -174,3 +174,37 @@ def test_greedy_generation_through_the_engine_and_scheduler(folders):
     for p, o in zip(prompts, outs):
         assert list(o.tokens) == model.greedy(p, 12)
     assert outs[5].cached_tokens >= 16
+
+
+def test_a_second_norm_without_a_feed_forward_is_applied_if_the_checkpoint_brings_one(folders, tmp_path):
+    """config.json does not say whether a layer without a feed-forward has a second norm: the
+    checkpoint does. Without the tensor the layer ends behind its first norm; with it, the
+    second norm is applied to alpha x alone."""
+    import shutil
+
+    from safetensors.torch import load_file, save_file
+
+    folder = tmp_path / "m"
+    shutil.copytree(folders["P"], folder)
+    tensors = load_file(str(folder / "model.safetensors"))
+    assert "l1.norm2" not in tensors
+    tensors["l1.norm2"] = (1.0 + 0.2 * torch.randn(96, generator=torch.Generator().manual_seed(1))).to(torch.bfloat16)
+    save_file(tensors, str(folder / "model.safetensors"))
+    _, cfg, _ = read_model_dir(folder)
+    assert cfg.layers[1].lone_second_norm and not cfg.layers[0].lone_second_norm
+    assert not read_model_dir(folders["P"])[1].layers[1].lone_second_norm
+    toks = np.random.default_rng(3).integers(0, 120, 30).tolist()
+    model = plain.PlainRadivik(folder)
+    pos, kept = np.arange(len(toks)), {}
+    x = model.w["embed"][np.asarray(toks)]
+    for i, layer in enumerate(model.cfg["layers"]):
+        x = plain.rms_norm(model.alpha * x + model.mixer(i, x, pos, kept), model.w[f"l{i}.norm1"], model.eps)
+        if layer["mlp"] is not None:
+            x = plain.rms_norm(model.alpha * x + model.feed_forward(i, x), model.w[f"l{i}.norm2"], model.eps)
+        elif i == 1:
+            x = plain.rms_norm(model.alpha * x, model.w["l1.norm2"], model.eps)
+    want = plain.rms_norm(x, model.w["final.norm"], model.eps) @ model.w["head"].T
+    rp = TraceReplayer(runner_for(folder, 8))
+    got = rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": toks, "want": list(range(30))}], "end": ["a"]})
+    assert np.abs(got - want).max() < 2e-5 * np.abs(want).max()
+    assert np.abs(got - model.logits(toks)).max() > 1e-3 * np.abs(want).max()      # and it is not a no-op
