@@ -16,6 +16,7 @@ import traces
 from emulated_ops import EmulatedOps
 from plain import radivik_plain as plain
 from prefixserve_amd.config import RadivikConfig, UnsupportedModelError, read_model_dir
+from prefixserve_amd.engine.batch import StepItem
 from prefixserve_amd.engine.replay import TraceReplayer
 from prefixserve_amd.engine.runner import ModelRunner
 from prefixserve_amd.models.radivik import build_radivik_spec
@@ -151,8 +152,7 @@ def test_layers_follow_the_plain_model_one_by_one(folders):
             return out
 
         blk.forward = forward
-    runner.step(TraceReplayer(runner) and [__import__("prefixserve_amd.engine.batch", fromlist=["StepItem"]).StepItem(
-        key="a", tokens=toks, start=0, block_tables=[[0, 1]], slot=0, want=[20])])
+    runner.step([StepItem(key="a", tokens=toks, start=0, block_tables=[[0, 1]], slot=0, want=[20])])
     assert len(seen) == len(want)
     for i, (got, exp) in enumerate(zip(seen, want)):
         assert np.abs(got - exp).max() < 2e-5 * np.abs(exp).max(), f"layer {i}"
