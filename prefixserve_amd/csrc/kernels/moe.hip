@@ -415,16 +415,25 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       }
     const bool more = k0 + kGroupBK < K;
     if (more) ask(k0 + kGroupBK);               // in flight while this round is multiplied
+    // The pairs' operand of every step is read from LDS two steps ahead of the matrix instructions
+    // that use it (read right in front of them, every group of four waited for its operand first).
+    const bf16_t* bsrc = as[buf] + r * kGroupLD + 8 * g;
+    auto b_of = [&](int step) {
+      return *reinterpret_cast<const bf16x8*>(bsrc + (step % MT) * 16 * kGroupLD + (step / MT) * 32);
+    };
+    bf16x8 bq[3];
+    bq[0] = b_of(0);
+    if (KK * MT > 1) bq[1] = b_of(1);
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
+    for (int step = 0; step < KK * MT; ++step) {
+      const int kk = step / MT, mt = step % MT;
+      if (step + 2 < KK * MT) bq[(step + 2) % 3] = b_of(step + 2);
+      __builtin_amdgcn_sched_barrier(0);        // the read stays in front of this step's matrix instructions
+      const bf16x8 b = bq[step % 3];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 b = *reinterpret_cast<const bf16x8*>(as[buf] + (mt * 16 + r) * kGroupLD + kk * 32 + 8 * g);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          acc_g[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca[kk][rt], b, acc_g[rt][mt], 0, 0, 0);
-          if (GATED) acc_u[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb[kk][rt], b, acc_u[rt][mt], 0, 0, 0);
-        }
+      for (int rt = 0; rt < RT; ++rt) {
+        acc_g[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca[kk][rt], b, acc_g[rt][mt], 0, 0, 0);
+        if (GATED) acc_u[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb[kk][rt], b, acc_u[rt][mt], 0, 0, 0);
       }
     }
     if (more) stage(buf ^ 1);                   // nobody reads that buffer: all passed the last barrier after reading it
