@@ -503,8 +503,9 @@ __global__ void to_activation_kernel(const float* __restrict__ in, A* __restrict
 
 // ------------------------------------------------------------------ rope + unit norm + kv append
 
-// One wave per (token, head) of a row [hq q heads | hkv k heads | hkv v heads] x d. A q or k head
-// is rotated (pair (i, i + d/2), table [pos][i] = (cos, sin); NULL: not rotated), then, with
+// A group of L lanes per (token, head) of a row [hq q heads | hkv k heads | hkv v heads] x d, L the
+// power of two that holds d/2 pairs (at most a wave: several heads share a wave when d < 128). A q
+// or k head is rotated (pair (i, i + d/2), table [pos][i] = (cos, sin); NULL: not rotated), then, with
 // norm_dim > 0, divided by sqrt(sum of squares / norm_dim + eps): the root mean square over the
 // norm_dim dimensions that are the head's own when the rest of its d slots hold zeros. The
 // result goes back into the row and, for a k head, to its page as a [16, d] row; a v head goes
@@ -513,10 +514,12 @@ template <typename A>
 __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     A* __restrict__ qkv, int hq, int hkv, int d, const int32_t* __restrict__ positions,
     const float2* __restrict__ table, int norm_dim, float eps, A* __restrict__ kv,
-    const int32_t* __restrict__ write_slot) {
+    const int32_t* __restrict__ write_slot, int group_lanes) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & (kWave - 1);
-  const int head = static_cast<int>(blockIdx.y) * 4 + static_cast<int>(threadIdx.x >> 6);
+  const int per_wave = kWave / group_lanes;
+  const int l = lane & (group_lanes - 1);
+  const int head = (static_cast<int>(blockIdx.y) * 4 + static_cast<int>(threadIdx.x >> 6)) * per_wave + lane / group_lanes;
   if (head >= hq + 2 * hkv) return;
   const int half = d >> 1;
   A* row = qkv + t * (static_cast<int64_t>(hq + 2 * hkv) * d) + static_cast<int64_t>(head) * d;
@@ -533,8 +536,8 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     float a[2], b[2];
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int i = lane + j * kWave;
+    for (int j = 0; j < 2; ++j) {                      // group_lanes = 64 when d > 128: two pairs per lane
+      const int i = l + j * group_lanes;
       a[j] = b[j] = 0.f;
       if (i < half) {
         const float u = to_float<A>(row[i]), v = to_float<A>(row[i + half]);
@@ -546,12 +549,16 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
       }
     }
     float inv = 1.f;
-    if (norm_dim > 0) inv = rsqrtf(wave_sum(ss) / static_cast<float>(norm_dim) + eps);
+    if (norm_dim > 0) {
+      // the sum over the head's group of lanes: partners of every step lie inside the group
+      for (int o = group_lanes >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+      inv = rsqrtf(ss / static_cast<float>(norm_dim) + eps);
+    }
     A* dst = (kv != nullptr && head >= hq)
                  ? kv + page * page_elems + (static_cast<int64_t>(head - hq) * kPage + off) * d : nullptr;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int i = lane + j * kWave;
+      const int i = l + j * group_lanes;
       if (i < half) {
         const A lo = from_float<A>(a[j] * inv), hi = from_float<A>(b[j] * inv);
         row[i] = lo;
@@ -565,7 +572,7 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
   } else if (kv != nullptr) {
     const int vh = head - hq - hkv;
     A* vpage = kv + page * page_elems + static_cast<int64_t>(hkv) * kPage * d + off;
-    for (int c = lane; c < d; c += kWave) vpage[(static_cast<int64_t>(vh) * d + c) * kPage] = row[c];
+    for (int c = l; c < d; c += group_lanes) vpage[(static_cast<int64_t>(vh) * d + c) * kPage] = row[c];
   }
 }
 
@@ -760,13 +767,19 @@ int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t to
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float2* tab = reinterpret_cast<const float2*>(table);
-  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(ceil_div(hq + 2 * hkv, 4)));
+  int group_lanes = 1;                                   // lanes per head: the power of two that holds d/2 pairs, up to a wave
+  while (group_lanes < 64 && group_lanes < head_dim / 2) group_lanes *= 2;
+  const int heads_per_block = 4 * (64 / group_lanes);
+  PSAMD_REQUIRE(ceil_div(hq + 2 * hkv, heads_per_block) <= 65535, "too many heads for one launch");
+  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(ceil_div(hq + 2 * hkv, heads_per_block)));
   if (act_dtype == kBF16) {
     rope_norm_kv_append_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim, positions,
-                                                                 tab, norm_dim, eps, static_cast<bf16_t*>(kv), write_slot);
+                                                                 tab, norm_dim, eps, static_cast<bf16_t*>(kv), write_slot,
+                                                                 group_lanes);
   } else if (act_dtype == kF32) {
     rope_norm_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<float*>(qkv), hq, hkv, head_dim, positions,
-                                                                tab, norm_dim, eps, static_cast<float*>(kv), write_slot);
+                                                                tab, norm_dim, eps, static_cast<float*>(kv), write_slot,
+                                                                group_lanes);
   } else {
     return fail("psamd_rope_norm_kv_append: activation dtype must be float32 or bfloat16");
   }
