@@ -131,6 +131,8 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 // part_o [32 * n_tiles * hq * nsplit * head_dim] and part_ml [32 * n_tiles * hq * nsplit * 2] carry
 // to a merge kernel.
 int psamd_attention_prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head_dim);
+// exact_weights (here and in psamd_attention_decode): the softmax weights enter the second product
+// as three bfloat16 terms whose sum is the float32 weight exactly, instead of rounded to bfloat16.
 // pf_tiles: (item, first query) of every tile of 32 queries; pf_blocks: the first tile of every run
 // of up to four consecutive tiles of one item, in the order of the tiles (n_blocks = 0: no such
 // list; steps with one or two query heads per kv head then run a slower form).
@@ -140,7 +142,7 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
                             const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                             const int32_t* item_start, const int32_t* item_pos0,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
-                            float scale, int window, float* part_o, float* part_ml, int nsplit);
+                            float scale, int window, float* part_o, float* part_ml, int nsplit, int exact_weights);
 
 // The plan for a decode step's keys: whether its context lengths count as skewed (one far longer
 // than the rest), into how many runs of at least how many keys each request's keys are cut, and
@@ -152,7 +154,8 @@ int psamd_attention_decode_max_parts(int max_requests);
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                            const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
-                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys);
+                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys,
+                           int exact_weights);
 
 // out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
 int64_t psamd_sample_scratch_floats(int rows);

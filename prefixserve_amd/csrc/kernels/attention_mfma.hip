@@ -73,13 +73,33 @@ constexpr int kMinSplitKeys = 512;   // a workgroup's share of a tile's keys is 
 // 4 waves take the 32-key tiles in turn and merge by log-sum-exp through LDS. Splitting the
 // keys (not the queries) over the waves keeps the longest dependent chain of tiles four
 // times shorter, which is what bounds a causal prompt's last rows.
+// A softmax weight as the second product's operand. Plain: rounded to bfloat16. P3: as the three
+// bfloat16 terms whose sum is the float32 weight exactly (8 + 8 + 8 bits of mantissa: each term is
+// the rounding of what the terms before it left), so that the weights enter the product as they
+// were computed in 32-bit; the product then takes three matrix instructions per operand of values.
+struct WeightTerms {
+  __bf16 hi, mid, lo;
+};
+template <bool P3>
+__device__ __forceinline__ WeightTerms split_weight(float p) {
+  WeightTerms w;
+  w.hi = static_cast<__bf16>(p);
+  w.mid = w.lo = static_cast<__bf16>(0.f);
+  if (P3) {
+    const float r1 = p - static_cast<float>(w.hi);
+    w.mid = static_cast<__bf16>(r1);
+    w.lo = static_cast<__bf16>(r1 - static_cast<float>(w.mid));
+  }
+  return w;
+}
+
 // Per wave the loop is unrolled by two with two register sets: the keys and values of the
 // wave's next tile are loaded before the current one is computed. The block table is staged
 // in LDS once (a page id fetched from global memory inside the loop would put a second,
 // unhidden latency in front of every tile's loads). Only tiles that touch the diagonal (or a
 // window's edge) pay for masking; the softmax uses exp2 with the scale folded into one
 // multiply-add per score.
-template <int NS>
+template <int NS, bool P3 = false>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
@@ -224,19 +244,27 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     }
     const float m_use = m == -INFINITY ? 0.f : m;
     float rowsum = 0.f;
-    bf16x8 pb[2];
+    bf16x8 pb[2], pm[2], pl[2];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -m_use));
       rowsum += p;
-      pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+      const WeightTerms w = split_weight<P3>(p);
+      pb[v >> 3][v & 7] = w.hi;
+      pm[v >> 3][v & 7] = w.mid;
+      pl[v >> 3][v & 7] = w.lo;
     }
     l += rowsum + __shfl_xor(rowsum, 32, kWave);
 #pragma unroll
     for (int cpage = 0; cpage < 2; ++cpage)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt) {
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pb[cpage], o[dt], 0, 0, 0);
+        if (P3) {
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pm[cpage], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pl[cpage], o[dt], 0, 0, 0);
+        }
+      }
   };
 
   {
@@ -348,7 +376,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // Measured and not kept: the scores of the next iteration issued before the softmax of the
 // current one (correct, no faster at head size 128, slower at 64 where it costs the second
 // workgroup per compute unit its registers), and the stores to LDS issued behind the barrier.
-template <int NS, int KT, int KP>
+template <int NS, int KT, int KP, bool P3 = false>
 __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_grouped_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
@@ -571,19 +599,27 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     float rowsum = 0.f;
 #pragma unroll
     for (int t = 0; t < KT; ++t) {
-      bf16x8 pb[2];
+      bf16x8 pb[2], pm[2], pl[2];
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const float p = __builtin_amdgcn_exp2f(fmaf(s[t][v], c, -m_use));
         rowsum += p;
-        pb[v >> 3][v & 7] = static_cast<__bf16>(p);
+        const WeightTerms w = split_weight<P3>(p);
+        pb[v >> 3][v & 7] = w.hi;
+        pm[v >> 3][v & 7] = w.mid;
+        pl[v >> 3][v & 7] = w.lo;
       }
 #pragma unroll
       for (int cpage = 0; cpage < 2; ++cpage)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
           const bf16_t* vr = vd + ((2 * t + cpage) * D + min(32 * dt + col, D - 1)) * VS;
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join(ld4(vr), ld4(vr + 8)), pb[cpage], o[dt], 0, 0, 0);
+          const bf16x8 vv = join(ld4(vr), ld4(vr + 8));
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, pb[cpage], o[dt], 0, 0, 0);
+          if (P3) {
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, pm[cpage], o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, pl[cpage], o[dt], 0, 0, 0);
+          }
         }
     }
     l += rowsum + __shfl_xor(rowsum, 32, kWave);
@@ -760,7 +796,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(
 
 // NS = D / 16, CT = ceil(group / 16) column tiles of query heads.
 // part_o[dec][head][split][D], part_ml[dec][head][split][2] = (max, sum).
-template <int NS, int CT>
+template <int NS, int CT, bool P3 = false>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ qkv, int q_stride, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ dec_items,
@@ -902,12 +938,15 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __expf(m[ct] - m_use);
       float rowsum = 0.f;
-      bf16x8 pb;
+      bf16x8 pb, pm, pl;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float p = __expf(sv[e] - m_use);
         rowsum += p;
-        pb[e] = static_cast<__bf16>(p);
+        const WeightTerms w = split_weight<P3>(p);
+        pb[e] = w.hi;
+        pm[e] = w.mid;
+        pl[e] = w.lo;
       }
       rowsum += __shfl_xor(rowsum, 16, kWave);
       rowsum += __shfl_xor(rowsum, 32, kWave);
@@ -917,6 +956,10 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       for (int ds = 0; ds < NS; ++ds) {
         o[ct][ds] *= alpha;
         o[ct][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[ds], pb, o[ct][ds], 0, 0, 0);
+        if (P3) {
+          o[ct][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[ds], pm, o[ct][ds], 0, 0, 0);
+          o[ct][ds] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[ds], pl, o[ct][ds], 0, 0, 0);
+        }
       }
     }
   }
@@ -1118,7 +1161,7 @@ static int prefill_nsplit(int n_tiles, int max_kv_len, int hq, int hkv, int head
   return per_head_nsplit(n_tiles, max_kv_len, hq);
 }
 
-template <int NS>
+template <int NS, bool P3>
 static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* out, const void* kv,
                           const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                           const int32_t* item_start, const int32_t* item_pos0,
@@ -1146,8 +1189,8 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
 #define PSAMD_GROUPED(KP_)                                                                                         \
   {                                                                                                               \
     const size_t smem = grouped_smem(16 * NS, 1, KP_, table_pages);                                               \
-    if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_>, smem)) {                                             \
-      attn_prefill_grouped_kernel<NS, 1, KP_><<<grid, dim3(256 * KP_), smem, s>>>(                                \
+    if (lds_allowed(attn_prefill_grouped_kernel<NS, 1, KP_, P3>, smem)) {                                         \
+      attn_prefill_grouped_kernel<NS, 1, KP_, P3><<<grid, dim3(256 * KP_), smem, s>>>(                            \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
           pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window,   \
           part_o, part_ml, pair, tiles_per_wg, pf_blocks, n_blocks);                                              \
@@ -1164,7 +1207,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
     PSAMD_GROUPED(1)
 #undef PSAMD_GROUPED
   }
-  attn_prefill_mfma_kernel<NS><<<dim3(hq, n_tiles, nsplit), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
+  attn_prefill_mfma_kernel<NS, P3><<<dim3(hq, n_tiles, nsplit), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
       item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml);
   const int rc = check_launch("psamd_attention_prefill");
@@ -1172,7 +1215,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
   return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);
 }
 
-template <int NS, int CT>
+template <int NS, int CT, bool P3>
 static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out, float* part_o,
                          float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start, const int32_t* item_end,
                          const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int nsplit, float scale,
@@ -1180,19 +1223,19 @@ static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const voi
   const int group = hq / hkv;
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * 16 * NS);
   const int64_t groups_of_8 = ceil_div(static_cast<int64_t>(n_dec) * nsplit, 8);
-  attn_decode_mfma_kernel<NS, CT><<<dim3(8 * hkv, static_cast<unsigned>(groups_of_8)), dim3(256), smem, s>>>(
+  attn_decode_mfma_kernel<NS, CT, P3><<<dim3(8 * hkv, static_cast<unsigned>(groups_of_8)), dim3(256), smem, s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), static_cast<bf16_t*>(out), part_o,
       part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles, n_dec);
   return check_launch("psamd_attention_decode");
 }
 
-template <int NS>
+template <int NS, bool P3>
 static int dispatch_decode_ct(int ct, hipStream_t s, const void* qkv, int q_stride, const void* kv, void* out,
                               float* part_o, float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                               const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
                               int hkv, int nsplit, float scale, int window, int min_tiles) {
 #define PSAMD_DEC(CT_)                                                                                             \
-  return launch_decode<NS, CT_>(s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
+  return launch_decode<NS, CT_, P3>(s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start, item_end, \
                                 table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles)
   switch (ct) {
     case 1: PSAMD_DEC(1);
@@ -1250,7 +1293,8 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
                             const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks, int max_kv_len,
                             const int32_t* item_start,
                             const int32_t* item_pos0, const int32_t* table_off, const int32_t* block_ids, int hq,
-                            int hkv, int head_dim, float scale, int window, float* part_o, float* part_ml, int nsplit) {
+                            int hkv, int head_dim, float scale, int window, float* part_o, float* part_ml, int nsplit,
+                            int exact_weights) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
   PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 8192 * kPage, "context too long for the block table staged in LDS");
@@ -1262,8 +1306,13 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
   PSAMD_REQUIRE(nsplit == 1 || (part_o != nullptr && part_ml != nullptr), "split keys need part_o and part_ml");
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define PSAMD_PF(NS_)                                                                                           \
-  return launch_prefill<NS_>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, max_kv_len, item_start, \
-                             item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml, nsplit)
+  return exact_weights                                                                                          \
+             ? launch_prefill<NS_, true>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, max_kv_len,  \
+                                         item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, \
+                                         part_ml, nsplit)                                                       \
+             : launch_prefill<NS_, false>(s, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, max_kv_len, \
+                                          item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, \
+                                          part_ml, nsplit)
   switch (head_dim / 16) {
     case 1: PSAMD_PF(1);
     case 2: PSAMD_PF(2);
@@ -1320,7 +1369,8 @@ int psamd_attention_decode_max_parts(int max_requests) { return std::max({4096, 
 int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
                            float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
                            const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
-                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys) {
+                           int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys,
+                           int exact_weights) {
   PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
   PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
   PSAMD_REQUIRE(nsplit >= 1 && nsplit <= 64, "nsplit must be in [1, 64]");
@@ -1333,8 +1383,12 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
   const int ct = group <= 16 ? 1 : (group <= 32 ? 2 : 4);
   int rc;
 #define PSAMD_DEC_NS(NS_)                                                                                          \
-  rc = dispatch_decode_ct<NS_>(ct, s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, item_start,    \
-                               item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles);       \
+  rc = exact_weights ? dispatch_decode_ct<NS_, true>(ct, s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec,  \
+                                                     item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, \
+                                                     window, min_tiles)                                          \
+                     : dispatch_decode_ct<NS_, false>(ct, s, qkv, q_stride, kv, out, part_o, part_ml, dec_items, n_dec, \
+                                                      item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, \
+                                                      window, min_tiles);                                        \
   break
   switch (head_dim / 16) {
     case 1: PSAMD_DEC_NS(1);

@@ -65,9 +65,9 @@ _SIGNATURES = {
     "psamd_attention_decode_plan": [_i32, _i32, _i32, _i32, _i32, _vp, _vp],
     "psamd_attention_decode_max_parts": [_i32],
     "psamd_attention_prefill": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
-                                _f32, _i32, _vp, _vp, _i32],
+                                _f32, _i32, _vp, _vp, _i32, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
-                               _i32, _f32, _i32, _i32],
+                               _i32, _f32, _i32, _i32, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
     "psamd_scaled_add_rmsnorm": [_vp, _vp, _f32, _vp, _i32, _i32, _i64, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
@@ -575,7 +575,10 @@ class HipOps:
         return bool(self.lib.psamd_attention_mfma_supports(hq, hkv, d))
 
     def paged_attention(self, qkv, out, kv, ctx, group: int, hq: int, hkv: int, d: int, scale: float,
-                        window: int | None) -> None:
+                        window: int | None, exact_weights: bool = False) -> None:
+        """``exact_weights``: the softmax weights enter the product with the values as computed in
+        32-bit (the matrix-core kernels then take them as three bfloat16 terms that sum to the float32
+        weight exactly) instead of rounded to bfloat16; the 32-bit kernels always do."""
         t = qkv.shape[0]
         g = ctx.groups[group]
         self._need(out.shape == (t, hq * d) and out.is_contiguous() and out.dtype == qkv.dtype, "attention: output")
@@ -605,7 +608,8 @@ class HipOps:
                     ctx.num_prefill_tiles, ctx.pf_blocks.data_ptr(), ctx.num_prefill_blocks, kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
                     g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win,
-                    part_o.data_ptr() if nsplit > 1 else None, part_ml.data_ptr() if nsplit > 1 else None, nsplit))
+                    part_o.data_ptr() if nsplit > 1 else None, part_ml.data_ptr() if nsplit > 1 else None, nsplit,
+                    int(exact_weights)))
             if ctx.num_decode:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
                 skewed = self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed
@@ -621,7 +625,7 @@ class HipOps:
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
                     ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(),
                     ctx.item_end.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale,
-                    win, min_run))
+                    win, min_run, int(exact_weights)))
             return
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),

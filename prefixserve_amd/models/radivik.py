@@ -46,7 +46,7 @@ def build_radivik_spec(cfg: RadivikConfig) -> ModelSpec:
         mixer = PartSpec("paged_attention", {
             "num_heads": m.heads, "num_kv_heads": m.kv_heads, "head_dim": m.dim, "value_dim": m.vdim,
             "names": MIXER_NAMES, "position": name, "scale": m.scale, "qk_norm_eps": cfg.norm_eps,
-            "own_kv": m.kv_from is None,
+            "own_kv": m.kv_from is None, "exact_weights": True,
         })
         ff = ff_norm = None
         if layer.mlp is not None:

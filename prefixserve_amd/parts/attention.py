@@ -70,12 +70,14 @@ class PagedAttention(Mixer):
       square over ``head_dim`` (no weight, eps inside the root), in 32-bit, before the key goes
       to its page.
     * ``own_kv`` False: the layer has no key and value projections; its run reads the cache
-      entry another run writes (``LayerRun.writes_cache`` False) with queries of its own."""
+      entry another run writes (``LayerRun.writes_cache`` False) with queries of its own.
+    * ``exact_weights``: the softmax weights enter the product with the values as they were computed
+      in 32-bit instead of rounded to the activation dtype."""
 
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], num_heads: int,
                  num_kv_heads: int, head_dim: int, names: Mapping[str, str], position: str | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
-                 qk_norm_eps: float | None = None, own_kv: bool = True) -> None:
+                 qk_norm_eps: float | None = None, own_kv: bool = True, exact_weights: bool = False) -> None:
         if num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads not divisible by {num_kv_heads} kv heads")
         self.hidden_size = int(hidden_size)
@@ -83,6 +85,7 @@ class PagedAttention(Mixer):
         self.value_dim = self.head_dim if value_dim is None else int(value_dim)
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.own_kv = bool(own_kv)
+        self.exact_weights = bool(exact_weights)
         self.names = dict(names)
         self.window = None if window is None else int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
@@ -172,8 +175,12 @@ class PagedAttention(Mixer):
                                     cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
                                     self.head_dim if self.qk_norm_eps is not None else 0, self.qk_norm_eps or 0.0)
         out = ws.get("attn.out", (t, self.q_size), rt.dtype)
-        ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
-                            self.slots, self.scale, cache.window)
+        if self.exact_weights:
+            ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
+                                self.slots, self.scale, cache.window, exact_weights=True)
+        else:
+            ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
+                                self.slots, self.scale, cache.window)
         return ops.linear_to_residual(out, self.w_o, "attn.delta", getattr(ctx, "residual", None))
 
 

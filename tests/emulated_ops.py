@@ -137,7 +137,7 @@ class EmulatedOps:
         """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
         return x.repeat_interleave(rep, dim=1)
 
-    def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window) -> None:
+    def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window, exact_weights=False) -> None:
         g = ctx.groups[group]
         t = qkv.shape[0]
         q = qkv[:, : hq * d].view(t, hq, d).float()

@@ -461,3 +461,47 @@ def test_the_command_line_on_a_radivik_folder(tmp_path):
         out = json.loads(proc.stdout.strip().splitlines()[-1])
         assert len(out["outputs"][0]["tokens"]) == 6 and out["outputs"][0]["finish_reason"] == "length"
     assert out["outputs"][0]["tokens"] == want
+
+
+@pytest.mark.parametrize("hq,hkv,d", [(8, 2, 64), (4, 4, 128), (6, 2, 80)])
+def test_softmax_weights_enter_the_second_product_unrounded(ops, hq, hkv, d):
+    """With the same value row under every key, what a run of keys hands to the merge is that row
+    times the sum of the weights as the product saw them, beside the sum of the weights in 32-bit: in
+    float32, before any output is rounded. Their ratio is 1 to float32 rounding with ``exact_weights``
+    and off by the bfloat16 step over the root of the number of keys without. (Two long contexts, so
+    that the decode kernel cuts the keys into runs and writes partial results.)"""
+    from prefixserve_amd.engine.batch import GroupMeta, StepItem, StepPacker
+
+    blocks, old = 400, [3000, 2500]
+    gen = torch.Generator().manual_seed(hq + d)
+    vec = (torch.randn(hkv, d, generator=gen) + 3.0).to(torch.bfloat16).to(DEV)
+    pk = StepPacker(torch.device(DEV), [GroupMeta(blocks, None)], 10, 100000, 8, ops.PREFILL_TILE_Q, skew_rule=ops.decode_is_skewed)
+    kv = torch.zeros((blocks, 2, hkv, 16 * d), dtype=torch.bfloat16, device=DEV)
+    perm = torch.randperm(blocks, generator=gen).tolist()
+    items = []
+    for i, o in enumerate(old):
+        table = [perm.pop() for _ in range(-(-(o + 1) // 16))]
+        pos = torch.arange(o + 1)
+        pg = torch.tensor(table)[pos // 16].to(DEV)
+        kv[:, 0].view(blocks, hkv, 16, d)[pg, :, (pos % 16).to(DEV), :] = rnd(o + 1, hkv, d, dtype=torch.bfloat16, seed=50 + i, scale=0.5)
+        kv[:, 1].view(blocks, hkv, d, 16)[pg, :, :, (pos % 16).to(DEV)] = vec
+        items.append(StepItem(i, [1], o, [table], slot=i))
+    ctx = pk.pack(items)
+    qkv = rnd(2, (hq + 2 * hkv) * d, dtype=torch.bfloat16, seed=77)
+    want = vec.float().repeat_interleave(hq // hkv, 0)                                 # [hq, d]
+    off = {}
+    for exact in (False, True):
+        out = torch.empty(2, hq * d, dtype=torch.bfloat16, device=DEV)
+        ops.paged_attention(qkv, out, kv, ctx, 0, hq, hkv, d, 1.0 / d ** 0.5, None, exact_weights=exact)
+        assert rel(out.view(2, hq, d), want[None].expand(2, hq, d)) < 4e-3         # the softmax weights sum to 1
+        nsplit, _ = ops.decode_plan(2, ctx.max_kv_len, ctx.decode_skewed, hkv, 0)
+        assert nsplit >= 2
+        rows = 2 * hq * nsplit                                                      # (request, head, run)
+        part_o = ops.ws._bufs["attn.part_o"][: rows * d].view(2, hq, nsplit, d)
+        total = ops.ws._bufs["attn.part_ml"][: rows * 2].view(2, hq, nsplit, 2)[..., 1]
+        used = total > 0.5                                                          # runs that held keys in this step
+        assert int(used.sum()) >= 4 * hq
+        ratio = (part_o / want[None, :, None, :]).mean(-1) / total.clamp_min(1e-30)
+        off[exact] = float((ratio[used] - 1.0).abs().max())
+    print(hq, hkv, d, off)
+    assert off[True] < 3e-6 and off[False] > 10 * off[True]
