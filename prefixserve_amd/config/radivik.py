@@ -151,7 +151,7 @@ class RadivikConfig:
                 raise UnsupportedModelError(f"layers[{i}] reads layer {j}'s keys and values but has other sizes")
         return cls(int(raw["vocab"]), int(raw["width"]), float(raw["norm"]["eps"]), float(raw["postln_alpha"]), tuple(layers))
 
-    def fitted_to_checkpoint(self, names: frozenset[str]) -> "RadivikConfig":
+    def fitted_to_checkpoint(self, names: "Mapping[str, tuple[int, ...]] | frozenset[str]") -> "RadivikConfig":
         """The configuration with what the checkpoint's tensor names decide."""
         layers = tuple(replace(layer, lone_second_norm=layer.mlp is None and f"l{i}.norm2" in names)
                        for i, layer in enumerate(self.layers))

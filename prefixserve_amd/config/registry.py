@@ -64,8 +64,8 @@ def read_model_dir(model_dir: str | Path) -> tuple[Architecture, Any, dict[str, 
     gen = json.loads(gen_path.read_text()) if gen_path.exists() else {}
     arch = architecture_of(raw)
     cfg = arch.config_cls.from_dicts(raw, gen)
-    # A configuration class may look at which tensors the checkpoint holds (names only, from the
-    # files' headers) where its config.json leaves something to the checkpoint.
+    # A configuration class may look at which tensors the checkpoint holds (names and shapes, from
+    # the files' headers) where its config.json leaves something to the checkpoint.
     fit = getattr(cfg, "fitted_to_checkpoint", None)
     if fit is not None:
         names = _tensor_names(model_dir)
@@ -74,16 +74,16 @@ def read_model_dir(model_dir: str | Path) -> tuple[Architecture, Any, dict[str, 
     return arch, cfg, raw
 
 
-def _tensor_names(model_dir: Path) -> frozenset[str] | None:
-    """Names of the tensors in the folder's safetensors files, read from their headers; None if there are none."""
+def _tensor_names(model_dir: Path) -> dict[str, tuple[int, ...]] | None:
+    """Name -> shape of the tensors in the folder's safetensors files, read from their headers; None if there are none."""
     import struct
 
     files = sorted(model_dir.glob("*.safetensors"))
     if not files:
         return None
-    names: set[str] = set()
+    names: dict[str, tuple[int, ...]] = {}
     for f in files:
         with open(f, "rb") as fh:
             (n,) = struct.unpack("<Q", fh.read(8))
-            names.update(k for k in json.loads(fh.read(n)) if k != "__metadata__")
-    return frozenset(names)
+            names.update((k, tuple(v["shape"])) for k, v in json.loads(fh.read(n)).items() if k != "__metadata__")
+    return names

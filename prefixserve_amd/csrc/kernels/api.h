@@ -25,8 +25,8 @@ int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delt
                       int64_t partial_stride, const int32_t* rows, const void* weight, int weight_dtype, float eps,
                       void* out, int act_dtype, int64_t out_rows, int hidden);
 
-// out[t, c] = silu(gate_up[t, c]) * gate_up[t, inter + c]
-int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter);
+// out[t, c] = act(gate_up[t, c]) * gate_up[t, inter + c]; gate: 0 = SiLU, 1 = ReLU, 2 = GELU (tanh form).
+int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter, int gate);
 
 // Rotates the q and k heads of qkv[t] in place by table[positions[t]] (NULL table: no rotation) and, if kv
 // is given, writes k and v of token t to page slot write_slot[t] (= page * 16 + offset).
@@ -48,6 +48,59 @@ int psamd_to_activation(void* stream, const float* in, void* out, int act_dtype,
 int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
                               const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
                               const int32_t* write_slot);
+
+// The general form of psamd_rope_norm_kv_append. bias (float [(hq + hkv) * head_dim] or NULL) is added to
+// the q and k heads first; q_weight / k_weight (float [head_dim] or NULL) multiply the heads behind the
+// division by the root mean square; v_from_k: rows are [q heads | k heads] only and the value written
+// to the pages is the k head as projected (with its bias, before rotation and norm).
+int psamd_qk_prepare_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                               const int32_t* positions, const float* table, int norm_dim, float eps, const float* bias,
+                               const float* q_weight, const float* k_weight, int v_from_k, void* kv,
+                               const int32_t* write_slot);
+
+// residual[r] += delta[r]; delta as for psamd_add_rmsnorm (one tensor in delta_dtype, or n_partials float32 slices).
+int psamd_residual_add(void* stream, float* residual, const void* delta, int delta_dtype, int n_partials,
+                       int64_t partial_stride, int64_t rows, int hidden);
+// x[r, c] = x[r, c] * factor + row[c] (row may be NULL) on a float32 tensor [rows, hidden].
+int psamd_stream_affine(void* stream, float* x, int64_t rows, int hidden, float factor, const float* row);
+// out[r] = [a[r], b[r]] in act_dtype, a and b float32 [rows, hidden].
+int psamd_concat_to_activation(void* stream, const float* a, const float* b, void* out, int act_dtype, int64_t rows,
+                               int hidden);
+
+// One small product per head: out[t, h, n] = sum_k x[t, h, k] * w[h, n, k], float accumulation. Row t of
+// x starts at x + t * x_row, its head h at + h * x_head (elements), likewise out; w is [H, N, K], dense.
+int psamd_heads_linear(void* stream, const void* x, int x_dtype, int64_t x_row, int x_head, const void* w, int w_dtype,
+                       void* out, int out_dtype, int64_t out_row, int out_head, int64_t M, int H, int N, int K);
+
+// Latent attention, one compressed vector per token. Row t of `in` is [hq heads x (dim + rot) | rank | rot]:
+// the compressed part is divided by its root mean square (eps inside the root) and multiplied by norm_w
+// (float [rank]), the shared key part and every head's last `rot` query dimensions are rotated pair by
+// pair, (2i, 2i + 1) by table[positions[t]][i] = (cos, sin). The page of kv ([blocks, 2, 1, 16 * slots])
+// gets the key [compressed | rotated part | zeros] and, transposed, the value [compressed | zeros];
+// q_lat[t, h] (slots wide) gets the rotated query part at [rank, rank + rot) and zeros behind it, and
+// is left alone in front: that is where the product of the head's other dimensions goes.
+int psamd_latent_kv_append(void* stream, const void* in, int64_t in_row, void* q_lat, int act_dtype, int64_t tokens,
+                           int hq, int dim, int rot, int rank, int slots, const int32_t* positions, const float* table,
+                           const float* norm_w, float eps, void* kv, const int32_t* write_slot);
+
+// A causal convolution per channel over each item's tokens, continued from the item's state:
+// u[t, c] = conv_b[c] + sum_j conv_w[c, j] * v(t - (taps - 1) + j, c) with v(s, c) = in[s, c] + in_bias[c]
+// for tokens of this step and the state's saved inputs (state[slot, (taps - 1) x width], oldest first)
+// in front of the item's first token. `in` rows are in_row apart. u is float32. The state is only read.
+int psamd_causal_conv(void* stream, const void* in, int act_dtype, int64_t in_row, const float* in_bias,
+                      const float* conv_w, const float* conv_b, float* u, const float* state, int64_t state_row,
+                      const int32_t* tok_item, const int32_t* item_start, const int32_t* slots, int64_t tokens,
+                      int width, int taps);
+
+// The gated linear recurrence over each item's tokens, state in 32-bit: with r = sigmoid(gates[t, b, c'] +
+// gate_b), i = sigmoid(gates[t, b, bw + c'] + gate_b) (gates [tokens, blocks, 2 * bw], c = b * bw + c'),
+// log a = decay[c] * r: S = a S + sqrt(1 - a^2) i u[t, c]; out[t, c] = S * gelu_tanh(y[t, c] + y_bias[c]).
+// S lives in state[slot, (taps - 1) * width + c]; behind the scan the state's saved inputs become the
+// item's last taps - 1 values of x[t, c] + x_bias[c].
+int psamd_gated_scan(void* stream, const float* gates, const float* gate_b, const float* u, const float* decay,
+                     const void* y, const void* x, int act_dtype, int64_t in_row, const float* y_bias,
+                     const float* x_bias, void* out, float* state, int64_t state_row, const int32_t* item_start,
+                     const int32_t* slots, int items, int width, int blocks, int taps);
 
 // Mixture of experts. Router: z = x w_router^T in float (x in x_dtype, w_router float [E, K]), score =
 // sigmoid(z); chosen[t, :] = the top largest scores' experts (lower index among equals, largest
@@ -93,7 +146,8 @@ int psamd_gemm_lt(void* stream, const void* x, const void* w, void* out, int out
                   int use_workspace, int accumulate);
 
 
-// bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up.
+// bfloat16 product for M <= 64 on the matrix cores. epilogue 1: w = [gate; up], out = silu(gate) * up;
+// 2 and 3: the same with ReLU and with GELU (tanh form) on the gate.
 // ksplit > 1: out receives ksplit float32 partial sums [ksplit][M, n_out] (plain epilogue only).
 int psamd_linear_skinny_ksplit(int M, int n_out, int K);
 int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, int out_dtype, int M, int n_out, int K,
@@ -119,10 +173,12 @@ int psamd_qkv_rope_append_normed(void* stream, const float* resid, const void* n
                                  const void* w, void* qkv_out, int M, int K, int hq, int hkv, int head_dim,
                                  const int32_t* positions, const float* table, void* kv, const int32_t* write_slot);
 
+// sink (float [hq] or NULL): exp(sink[h]) is added to the softmax's denominator. dist_bias (float
+// [hq, n_dist] or NULL): dist_bias[h, min(i - j, n_dist - 1)] is added to the scaled score of query i and key j.
 int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* out, const void* kv, int act_dtype,
                             int64_t tokens, const int32_t* positions, const int32_t* tok_item,
                             const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
-                            float scale, int window);
+                            float scale, int window, const float* sink, const float* dist_bias, int n_dist);
 
 int psamd_attention_mfma_supports(int hq, int hkv, int head_dim);
 

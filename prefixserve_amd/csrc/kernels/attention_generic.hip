@@ -1,6 +1,9 @@
 // Causal grouped-query attention over the paged cache, the straightforward way: one wave
 // per (new token, query head), float arithmetic throughout, any head size that is a
-// multiple of 2 up to 256, any number of heads and groups, optional sliding window.
+// multiple of 2 up to 256, any number of heads and groups, optional sliding window, an optional
+// learned sink per head (a term exp(sink) in the softmax's denominator that has no key and no
+// value) and an optional bias on the scaled score that depends on the head and on how far back
+// the key lies (a table per head, its last entry standing for every larger distance).
 // It is the attention of the exact 32-bit path and the fallback for shapes the
 // matrix-core kernels do not take.
 //
@@ -17,7 +20,8 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const A* __restrict__ qkv, int q_stride, A* __restrict__ out, const A* __restrict__ kv,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_item,
     const int32_t* __restrict__ table_off, const int32_t* __restrict__ block_ids,
-    int hq, int hkv, int d, float scale, int window) {
+    int hq, int hkv, int d, float scale, int window, const float* __restrict__ sink,
+    const float* __restrict__ dist_bias, int n_dist) {
   __shared__ float q_s[256];
   __shared__ float p_s[kWave];
   __shared__ int32_t base_s[kWave];   // element offset of (page, kv head) for each key of the chunk
@@ -50,6 +54,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot = fmaf(q_s[i], to_float<A>(kr[i]), dot);
       s = dot * scale;
+      if (dist_bias != nullptr) s += dist_bias[static_cast<int64_t>(h) * n_dist + min(pos - j, n_dist - 1)];
       base_s[lane] = static_cast<int32_t>(page);
       off_s[lane] = off;
     }
@@ -76,6 +81,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     }
     __syncthreads();
   }
+  if (sink != nullptr) l += expf(sink[h] - m);     // the query's own key is always seen: m is finite
   const float inv = 1.f / l;
   A* o = out + t * (static_cast<int64_t>(hq) * d) + h * d;
 #pragma unroll
@@ -92,7 +98,9 @@ using namespace psamd;
 extern "C" int psamd_attention_generic(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
                                        int act_dtype, int64_t tokens, const int32_t* positions,
                                        const int32_t* tok_item, const int32_t* table_off, const int32_t* block_ids,
-                                       int hq, int hkv, int head_dim, float scale, int window) {
+                                       int hq, int hkv, int head_dim, float scale, int window, const float* sink,
+                                       const float* dist_bias, int n_dist) {
+  PSAMD_REQUIRE(dist_bias == nullptr || n_dist >= 1, "a distance bias needs at least one entry per head");
   PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv > 0 && hq % hkv == 0, "bad head counts");
   PSAMD_REQUIRE(head_dim > 0 && head_dim <= 256, "head_dim must be in [1, 256]");
   PSAMD_REQUIRE(hq <= 65535, "too many heads for one launch");
@@ -102,11 +110,11 @@ extern "C" int psamd_attention_generic(void* stream, const void* qkv, int q_stri
   if (act_dtype == kBF16) {
     attention_generic_kernel<bf16_t><<<grid, dim3(64), 0, s>>>(
         static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),
-        positions, tok_item, table_off, block_ids, hq, hkv, head_dim, scale, window);
+        positions, tok_item, table_off, block_ids, hq, hkv, head_dim, scale, window, sink, dist_bias, n_dist);
   } else if (act_dtype == kF32) {
     attention_generic_kernel<float><<<grid, dim3(64), 0, s>>>(
         static_cast<const float*>(qkv), q_stride, static_cast<float*>(out), static_cast<const float*>(kv),
-        positions, tok_item, table_off, block_ids, hq, hkv, head_dim, scale, window);
+        positions, tok_item, table_off, block_ids, hq, hkv, head_dim, scale, window, sink, dist_bias, n_dist);
   } else {
     return fail("psamd_attention_generic: activation dtype must be float32 or bfloat16");
   }

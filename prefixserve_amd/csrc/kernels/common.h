@@ -39,6 +39,18 @@ __device__ __forceinline__ float load_as_float(const void* p, int dtype, int64_t
   return dtype == kBF16 ? bf16_to_float(static_cast<const bf16_t*>(p)[i]) : static_cast<const float*>(p)[i];
 }
 
+// GELU in its tanh form: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// The activation on the gate of a gated feed-forward: 0 = SiLU, 1 = ReLU, 2 = GELU (tanh form).
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 1) return fmaxf(g, 0.f);
+  if (act == 2) return gelu_tanh_f(g);
+  return g / (1.f + __expf(-g));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

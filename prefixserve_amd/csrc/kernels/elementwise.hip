@@ -203,20 +203,20 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_vec8_kernel(
 // ------------------------------------------------------------------ swiglu
 
 template <typename A>
-__global__ void swiglu_kernel(const A* __restrict__ gate_up, A* __restrict__ out, int64_t tokens, int inter) {
+__global__ void swiglu_kernel(const A* __restrict__ gate_up, A* __restrict__ out, int64_t tokens, int inter, int act) {
   const int64_t n = tokens * inter;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t t = i / inter, c = i - t * inter;
     const float g = to_float<A>(gate_up[t * 2 * inter + c]);
     const float u = to_float<A>(gate_up[t * 2 * inter + inter + c]);
-    out[i] = from_float<A>(g / (1.f + __expf(-g)) * u);
+    out[i] = from_float<A>(gate_act(g, act) * u);
   }
 }
 
 // bfloat16, intermediate size a multiple of 8: 16-byte accesses, 8 elements per thread.
 __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int64_t tokens,
-                                   int inter) {
+                                   int inter, int act) {
   const int chunks = inter >> 3;
   const int64_t n = tokens * chunks;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
@@ -231,8 +231,8 @@ __global__ void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* _
     for (int k = 0; k < 4; ++k) {
       const float g0 = __uint_as_float(g4[k] << 16), g1 = __uint_as_float(g4[k] & 0xffff0000u);
       const float u0 = __uint_as_float(u4[k] << 16), u1 = __uint_as_float(u4[k] & 0xffff0000u);
-      pk[k] = static_cast<uint32_t>(float_to_bf16(g0 / (1.f + __expf(-g0)) * u0)) |
-              (static_cast<uint32_t>(float_to_bf16(g1 / (1.f + __expf(-g1)) * u1)) << 16);
+      pk[k] = static_cast<uint32_t>(float_to_bf16(gate_act(g0, act) * u0)) |
+              (static_cast<uint32_t>(float_to_bf16(gate_act(g1, act) * u1)) << 16);
     }
     *reinterpret_cast<uint4*>(out + t * inter + e) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
   }
@@ -514,15 +514,17 @@ template <typename A>
 __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     A* __restrict__ qkv, int hq, int hkv, int d, const int32_t* __restrict__ positions,
     const float2* __restrict__ table, int norm_dim, float eps, A* __restrict__ kv,
-    const int32_t* __restrict__ write_slot, int group_lanes) {
+    const int32_t* __restrict__ write_slot, int group_lanes, const float* __restrict__ bias,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, int v_from_k) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & (kWave - 1);
   const int per_wave = kWave / group_lanes;
   const int l = lane & (group_lanes - 1);
   const int head = (static_cast<int>(blockIdx.y) * 4 + static_cast<int>(threadIdx.x >> 6)) * per_wave + lane / group_lanes;
-  if (head >= hq + 2 * hkv) return;
+  const int row_heads = hq + (v_from_k ? hkv : 2 * hkv);
+  if (head >= row_heads) return;
   const int half = d >> 1;
-  A* row = qkv + t * (static_cast<int64_t>(hq + 2 * hkv) * d) + static_cast<int64_t>(head) * d;
+  A* row = qkv + t * (static_cast<int64_t>(row_heads) * d) + static_cast<int64_t>(head) * d;
   int64_t page = 0;
   int off = 0;
   if (kv != nullptr) {
@@ -533,6 +535,7 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
   const int64_t page_elems = 2LL * hkv * kPage * d;
   if (head < hq + hkv) {
     const int pos = positions[t];
+    const float* nw = head < hq ? q_weight : k_weight;
     float a[2], b[2];
     float ss = 0.f;
 #pragma unroll
@@ -540,7 +543,17 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
       const int i = l + j * group_lanes;
       a[j] = b[j] = 0.f;
       if (i < half) {
-        const float u = to_float<A>(row[i]), v = to_float<A>(row[i + half]);
+        float u = to_float<A>(row[i]), v = to_float<A>(row[i + half]);
+        if (bias != nullptr) {
+          u += bias[static_cast<int64_t>(head) * d + i];
+          v += bias[static_cast<int64_t>(head) * d + i + half];
+        }
+        if (v_from_k && head >= hq && kv != nullptr) {
+          // the value is the key as projected: before rotation and norm
+          A* vpage = kv + page * page_elems + static_cast<int64_t>(hkv) * kPage * d + off;
+          vpage[(static_cast<int64_t>(head - hq) * d + i) * kPage] = from_float<A>(u);
+          vpage[(static_cast<int64_t>(head - hq) * d + i + half) * kPage] = from_float<A>(v);
+        }
         float2 cs = float2{1.f, 0.f};
         if (table != nullptr) cs = table[static_cast<int64_t>(pos) * half + i];
         a[j] = u * cs.x - v * cs.y;
@@ -560,7 +573,8 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     for (int j = 0; j < 2; ++j) {
       const int i = l + j * group_lanes;
       if (i < half) {
-        const A lo = from_float<A>(a[j] * inv), hi = from_float<A>(b[j] * inv);
+        const A lo = from_float<A>(a[j] * inv * (nw != nullptr ? nw[i] : 1.f));
+        const A hi = from_float<A>(b[j] * inv * (nw != nullptr ? nw[i + half] : 1.f));
         row[i] = lo;
         row[i + half] = hi;
         if (dst != nullptr) {
@@ -573,6 +587,40 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     const int vh = head - hq - hkv;
     A* vpage = kv + page * page_elems + static_cast<int64_t>(hkv) * kPage * d + off;
     for (int c = l; c < d; c += group_lanes) vpage[(static_cast<int64_t>(vh) * d + c) * kPage] = row[c];
+  }
+}
+
+// ------------------------------------------------------------------ sums and copies of the stream
+
+// residual += delta, where delta is one tensor or n_partials float32 slices (summed in ascending order).
+template <typename DT>
+__global__ void residual_add_kernel(float* __restrict__ residual, const DT* __restrict__ delta, int n_partials,
+                                    int64_t partial_stride, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float x = residual[i];
+    for (int p = 0; p < n_partials; ++p) x += to_float<DT>(delta[p * partial_stride + i]);
+    residual[i] = x;
+  }
+}
+
+__global__ void stream_affine_kernel(float* __restrict__ x, int64_t n, int hidden, float factor,
+                                     const float* __restrict__ row) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const float add = row != nullptr ? row[i % hidden] : 0.f;
+    x[i] = x[i] * factor + add;
+  }
+}
+
+template <typename A>
+__global__ void concat_to_activation_kernel(const float* __restrict__ a, const float* __restrict__ b, A* __restrict__ out,
+                                            int64_t n, int hidden) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = i / hidden, c = i - r * hidden;
+    out[r * 2 * hidden + c] = from_float<A>(a[i]);
+    out[r * 2 * hidden + hidden + c] = from_float<A>(b[i]);
   }
 }
 
@@ -642,8 +690,9 @@ int psamd_add_rmsnorm(void* stream, float* residual, const void* delta, int delt
   return check_launch("psamd_add_rmsnorm");
 }
 
-int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter) {
+int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, int64_t tokens, int inter, int gate) {
   PSAMD_REQUIRE(tokens >= 0 && inter > 0, "bad sizes");
+  PSAMD_REQUIRE(gate >= 0 && gate <= 2, "the gate's activation is 0 (SiLU), 1 (ReLU) or 2 (GELU, tanh form)");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = tokens * inter;
@@ -651,13 +700,13 @@ int psamd_swiglu(void* stream, const void* gate_up, void* out, int act_dtype, in
   if (act_dtype == kBF16 && inter % 8 == 0) {
     const int vblocks = static_cast<int>(std::min<int64_t>(ceil_div(n / 8, 256), 65536));
     swiglu_vec8_kernel<<<dim3(vblocks), dim3(256), 0, s>>>(static_cast<const bf16_t*>(gate_up),
-                                                           static_cast<bf16_t*>(out), tokens, inter);
+                                                           static_cast<bf16_t*>(out), tokens, inter, gate);
   } else if (act_dtype == kBF16) {
     swiglu_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const bf16_t*>(gate_up),
-                                                            static_cast<bf16_t*>(out), tokens, inter);
+                                                            static_cast<bf16_t*>(out), tokens, inter, gate);
   } else if (act_dtype == kF32) {
     swiglu_kernel<float><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const float*>(gate_up),
-                                                           static_cast<float*>(out), tokens, inter);
+                                                           static_cast<float*>(out), tokens, inter, gate);
   } else {
     return fail("psamd_swiglu: activation dtype must be float32 or bfloat16");
   }
@@ -756,34 +805,92 @@ int psamd_to_activation(void* stream, const float* in, void* out, int act_dtype,
   return check_launch("psamd_to_activation");
 }
 
-int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
-                              const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
-                              const int32_t* write_slot) {
+int psamd_qk_prepare_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                               const int32_t* positions, const float* table, int norm_dim, float eps, const float* bias,
+                               const float* q_weight, const float* k_weight, int v_from_k, void* kv,
+                               const int32_t* write_slot) {
   PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv >= 0, "bad sizes");
   PSAMD_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256, "head_dim must be even and at most 256");
   PSAMD_REQUIRE(norm_dim >= 0 && norm_dim <= head_dim, "norm_dim must be in [0, head_dim]");
   PSAMD_REQUIRE(kv == nullptr || (write_slot != nullptr && hkv > 0), "a cache needs write slots and kv heads");
-  PSAMD_REQUIRE(tokens <= 2147483647LL && ceil_div(hq + 2 * hkv, 4) <= 65535, "too large for one launch");
+  PSAMD_REQUIRE(tokens <= 2147483647LL, "too large for one launch");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float2* tab = reinterpret_cast<const float2*>(table);
+  const int row_heads = hq + (v_from_k ? hkv : 2 * hkv);
   int group_lanes = 1;                                   // lanes per head: the power of two that holds d/2 pairs, up to a wave
   while (group_lanes < 64 && group_lanes < head_dim / 2) group_lanes *= 2;
   const int heads_per_block = 4 * (64 / group_lanes);
-  PSAMD_REQUIRE(ceil_div(hq + 2 * hkv, heads_per_block) <= 65535, "too many heads for one launch");
-  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(ceil_div(hq + 2 * hkv, heads_per_block)));
+  PSAMD_REQUIRE(ceil_div(row_heads, heads_per_block) <= 65535, "too many heads for one launch");
+  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(ceil_div(row_heads, heads_per_block)));
   if (act_dtype == kBF16) {
     rope_norm_kv_append_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim, positions,
                                                                  tab, norm_dim, eps, static_cast<bf16_t*>(kv), write_slot,
-                                                                 group_lanes);
+                                                                 group_lanes, bias, q_weight, k_weight, v_from_k);
   } else if (act_dtype == kF32) {
     rope_norm_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<float*>(qkv), hq, hkv, head_dim, positions,
                                                                 tab, norm_dim, eps, static_cast<float*>(kv), write_slot,
-                                                                group_lanes);
+                                                                group_lanes, bias, q_weight, k_weight, v_from_k);
   } else {
-    return fail("psamd_rope_norm_kv_append: activation dtype must be float32 or bfloat16");
+    return fail("psamd_qk_prepare_kv_append: activation dtype must be float32 or bfloat16");
   }
-  return check_launch("psamd_rope_norm_kv_append");
+  return check_launch("psamd_qk_prepare_kv_append");
+}
+
+int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
+                              const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
+                              const int32_t* write_slot) {
+  return psamd_qk_prepare_kv_append(stream, qkv, act_dtype, tokens, hq, hkv, head_dim, positions, table, norm_dim, eps,
+                                    nullptr, nullptr, nullptr, 0, kv, write_slot);
+}
+
+// residual[r] += delta[r] (delta as for psamd_add_rmsnorm: one tensor in delta_dtype or float32 slices).
+int psamd_residual_add(void* stream, float* residual, const void* delta, int delta_dtype, int n_partials,
+                       int64_t partial_stride, int64_t rows, int hidden) {
+  PSAMD_REQUIRE(rows >= 0 && hidden > 0 && n_partials >= 1 && delta != nullptr, "bad sizes");
+  PSAMD_REQUIRE(n_partials == 1 || delta_dtype == kF32, "partial sums are float32");
+  if (rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = rows * hidden;
+  const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
+  if (delta_dtype == kBF16) {
+    residual_add_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(residual, static_cast<const bf16_t*>(delta), n_partials,
+                                                                  partial_stride, n);
+  } else if (delta_dtype == kF32) {
+    residual_add_kernel<float><<<dim3(blocks), dim3(256), 0, s>>>(residual, static_cast<const float*>(delta), n_partials,
+                                                                 partial_stride, n);
+  } else {
+    return fail("psamd_residual_add: delta dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_residual_add");
+}
+
+// x[r, c] = x[r, c] * factor + (row != NULL ? row[c] : 0), in float32.
+int psamd_stream_affine(void* stream, float* x, int64_t rows, int hidden, float factor, const float* row) {
+  PSAMD_REQUIRE(rows >= 0 && hidden > 0, "bad sizes");
+  if (rows == 0) return 0;
+  const int64_t n = rows * hidden;
+  const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
+  stream_affine_kernel<<<dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(x, n, hidden, factor, row);
+  return check_launch("psamd_stream_affine");
+}
+
+// out[r] = [a[r], b[r]] in act_dtype: two float32 streams side by side as one product's input.
+int psamd_concat_to_activation(void* stream, const float* a, const float* b, void* out, int act_dtype, int64_t rows,
+                               int hidden) {
+  PSAMD_REQUIRE(rows >= 0 && hidden > 0, "bad sizes");
+  if (rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = rows * hidden;
+  const int blocks = static_cast<int>(std::min<int64_t>(ceil_div(n, 256), 65536));
+  if (act_dtype == kBF16) {
+    concat_to_activation_kernel<bf16_t><<<dim3(blocks), dim3(256), 0, s>>>(a, b, static_cast<bf16_t*>(out), n, hidden);
+  } else if (act_dtype == kF32) {
+    concat_to_activation_kernel<float><<<dim3(blocks), dim3(256), 0, s>>>(a, b, static_cast<float*>(out), n, hidden);
+  } else {
+    return fail("psamd_concat_to_activation: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_concat_to_activation");
 }
 
 }  // extern "C"

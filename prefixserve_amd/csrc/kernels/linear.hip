@@ -141,7 +141,9 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g)); }
+// The activation the gated epilogues apply to the gate (see gate_act), set by the entry points
+// for the launches they make.
+static thread_local int g_gate_act = 0;
 
 // *p += v, done by the memory side, nothing returned: the way K-slices of different workgroups,
 // on any die, add into one float32 sum.
@@ -178,7 +180,7 @@ constexpr int skinny_depth(int mt, int rt) { return mt == 1 ? 8 : (mt * rt <= 2 
 // the additions, and with it the last bit of the sums, differs from run to run.
 template <int MT, int RT, int WV, bool SWIGLU, bool SPLIT, typename TO, int U = skinny_depth(MT, RT), bool ATOMIC = false>
 __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                          TO* __restrict__ out, int M, int n_out, int K) {
+                                                          TO* __restrict__ out, int M, int n_out, int K, int act = 0) {
   constexpr int NACC = SWIGLU ? 2 * MT : MT;
   __shared__ f32x4 red[SPLIT ? WV : 1][NACC][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(64 * WV) void skinny_mfma_kernel(const bf16_t* __re
   auto finish = [&](int rt, int mt, f32x4 sum, f32x4 up) {
     if (SWIGLU) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+      for (int v = 0; v < 4; ++v) sum[v] = gate_act(sum[v], act) * up[v];
     }
     const int m = mt * 16 + r;
     if (m >= M) return;
@@ -404,7 +406,7 @@ __device__ __forceinline__ float stage_scale(const Tokens& tk, const float* ss, 
 // out[M][n_out] (see skinny_mfma_kernel).
 template <int RT, int ROWS, bool SWIGLU, typename TO, bool NORMED = false, bool ATOMIC = false>
 __global__ __launch_bounds__(512) void stream_kernel(Tokens tk, const bf16_t* __restrict__ w,
-                                                  TO* __restrict__ out, int M, int n_out, int K, int groups) {
+                                                  TO* __restrict__ out, int M, int n_out, int K, int groups, int act = 0) {
   constexpr int WV = 8, U = 8, NACC = SWIGLU ? 2 : 1;
   extern __shared__ __align__(16) unsigned char stream_smem[];
   const int steps_all = K >> 5;
@@ -490,7 +492,7 @@ __global__ __launch_bounds__(512) void stream_kernel(Tokens tk, const bf16_t* __
         for (int w2 = 1; w2 < WV; ++w2) up += red[((w2 * RT + rt) * NACC + 1) * 64 + lane];
         if (NORMED) up *= row_scale;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) sum[v] = silu_f(sum[v]) * up[v];
+        for (int v = 0; v < 4; ++v) sum[v] = gate_act(sum[v], act) * up[v];
       }
       if (r < M) {
         TO* dst = out + (static_cast<int64_t>(ATOMIC ? 0 : blockIdx.y) * M + r) * n_out;
@@ -531,7 +533,7 @@ static int launch_stream(hipStream_t s, const Tokens& tk, const void* w, void* o
       set_error("psamd_linear_skinny: " + std::to_string(smem) + " bytes of LDS were refused");
       return -1;
     }
-    kernel<<<grid, block, smem, s>>>(tk, wp, dst, M, n_out, K, groups);
+    kernel<<<grid, block, smem, s>>>(tk, wp, dst, M, n_out, K, groups, g_gate_act);
     return check_launch("psamd_linear_skinny");
   };
   if constexpr (ATOMIC) {
@@ -550,7 +552,7 @@ static int launch_skinny2(hipStream_t s, const void* x, const void* w, void* out
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   if constexpr (SWIGLU) {
-    skinny_mfma_kernel<MT, RT, WV, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
+    skinny_mfma_kernel<MT, RT, WV, true, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K, g_gate_act);
   } else if (out_dtype == kBF16) {
     skinny_mfma_kernel<MT, RT, WV, false, SPLIT, bf16_t><<<grid, block, 0, s>>>(xp, wp, static_cast<bf16_t*>(out), M, n_out, K);
   } else {
@@ -637,7 +639,7 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
     if (M > 8 && ceil_div(n_out, 16) >= 4 * 200) {
       const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(n_out, 16), 4)), 1u), block(64 * 8);
       skinny_mfma_kernel<MT, 4, 8, true, true, bf16_t, 1><<<grid, block, 0, s>>>(
-          static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K);
+          static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K, g_gate_act);
       return check_launch("psamd_linear_skinny");
     }
     if constexpr (MT == 1) {
@@ -646,7 +648,7 @@ static int launch_skinny1(hipStream_t s, const void* x, const void* w, void* out
       if (M > 8 && ceil_div(n_out, 16) >= 2 * 200) {
         const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(n_out, 16), 2)), 1u), block(64 * 8);
         skinny_mfma_kernel<1, 2, 8, true, true, bf16_t, 1><<<grid, block, 0, s>>>(
-            static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K);
+            static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), M, n_out, K, g_gate_act);
         return check_launch("psamd_linear_skinny");
       }
     }
@@ -962,7 +964,11 @@ int psamd_linear_skinny(void* stream, const void* x, const void* w, void* out, i
                         int epilogue, int ksplit) {
   PSAMD_REQUIRE(M >= 1 && M <= 64, "M must be in [1, 64]");
   PSAMD_REQUIRE(n_out > 0 && K > 0 && K % 8 == 0, "K must be a positive multiple of 8");
-  PSAMD_REQUIRE(epilogue == 0 || epilogue == 1, "unknown epilogue");
+  PSAMD_REQUIRE(epilogue >= 0 && epilogue <= 3, "unknown epilogue");
+  if (epilogue >= 1) {             // 1, 2, 3: the gated epilogue with SiLU, ReLU or GELU (tanh form) on the gate
+    g_gate_act = epilogue - 1;
+    epilogue = 1;
+  }
   PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "output must be bfloat16 or float32");
   PSAMD_REQUIRE(epilogue == 0 || out_dtype == kBF16, "the SwiGLU epilogue writes bfloat16");
   PSAMD_REQUIRE(ksplit >= 1 && ksplit <= 64, "ksplit must be in [1, 64]");
@@ -1035,7 +1041,11 @@ int psamd_linear_skinny_add(void* stream, const void* x, const void* w, float* o
 int psamd_linear_normed(void* stream, const float* resid, const int32_t* rows, const void* norm_w, int norm_w_dtype,
                         float eps, const void* w, void* out, int out_dtype, int M, int n_out, int K, int epilogue) {
   PSAMD_REQUIRE(normed_ok(M, K), "M must be in [1, 16] and K a multiple of 32 that fits in LDS");
-  PSAMD_REQUIRE(n_out > 0 && (epilogue == 0 || epilogue == 1), "bad sizes");
+  PSAMD_REQUIRE(n_out > 0 && epilogue >= 0 && epilogue <= 3, "bad sizes");
+  if (epilogue >= 1) {             // as in psamd_linear_skinny
+    g_gate_act = epilogue - 1;
+    epilogue = 1;
+  }
   PSAMD_REQUIRE(out_dtype == kBF16 || out_dtype == kF32, "output must be bfloat16 or float32");
   PSAMD_REQUIRE(epilogue == 0 || out_dtype == kBF16, "the SwiGLU epilogue writes bfloat16");
   PSAMD_REQUIRE(norm_w_dtype == kBF16 || norm_w_dtype == kF32, "the norm's weight is bfloat16 or float32");

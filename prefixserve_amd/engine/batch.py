@@ -86,6 +86,11 @@ class StepContext:
     # The stream's copy in the activation dtype when a block has just written one beside it
     # (a norm behind the sum does): the next block's sub-layer reads it instead of converting.
     stream_copy: Any = None
+    # The token table's output behind its transforms (float32 [T, hidden]), kept when a transform
+    # of the stream between layers needs it, and the pass through a repeated stretch of layers
+    # the run about to start belongs to.
+    embedding_output: Any = None
+    pass_index: int = 0
 
 
 class StepPacker:

@@ -46,7 +46,7 @@ logger = logging.getLogger(__name__)
 _SIGNATURES = {
     "psamd_embed": [_vp, _vp, _vp, _i32, _vp, _i64, _i32, _i32],
     "psamd_add_rmsnorm": [_vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
-    "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32],
+    "psamd_swiglu": [_vp, _vp, _vp, _i32, _i64, _i32, _i32],
     "psamd_rope_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
     "psamd_linear": [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i32],
     "psamd_gemm_lt": [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32],
@@ -57,7 +57,8 @@ _SIGNATURES = {
     "psamd_linear_skinny_add": [_vp, _vp, _vp, _vp, _i32, _i32, _i32],
     "psamd_linear_normed": [_vp, _vp, _vp, _vp, _i32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32],
     "psamd_qkv_rope_append_normed": [_vp, _vp, _vp, _i32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp],
-    "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32],
+    "psamd_attention_generic": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32,
+                                _vp, _vp, _i32],
     "psamd_attention_mfma_supports": [_i32, _i32, _i32],
     "psamd_attention_prefill_nsplit": [_i32, _i32, _i32, _i32, _i32],
     "psamd_attention_prefill_part_rows": [_i32, _i32, _i32],
@@ -72,6 +73,14 @@ _SIGNATURES = {
     "psamd_scaled_add_rmsnorm": [_vp, _vp, _f32, _vp, _i32, _i32, _i64, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
     "psamd_rope_norm_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp],
+    "psamd_qk_prepare_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp, _vp, _i32, _vp, _vp],
+    "psamd_residual_add": [_vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32],
+    "psamd_stream_affine": [_vp, _vp, _i64, _i32, _f32, _vp],
+    "psamd_concat_to_activation": [_vp, _vp, _vp, _vp, _i32, _i64, _i32],
+    "psamd_heads_linear": [_vp, _vp, _i32, _i64, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i64, _i32, _i32, _i32],
+    "psamd_latent_kv_append": [_vp, _vp, _i64, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _vp],
+    "psamd_causal_conv": [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32],
+    "psamd_gated_scan": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32, _i32, _i32, _i32],
     "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
     "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_moe_grouped_max_tiles": [_i64, _i32],
@@ -81,6 +90,9 @@ _SIGNATURES = {
 }
 
 
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
 class HipOps:
     PREFILL_TILE_Q = 32    # queries per workgroup of the prefill attention kernel (its 4 waves split the keys)
     SKINNY_MAX_ROWS = 64
@@ -88,6 +100,7 @@ class HipOps:
     LIBRARY_ADD_MIN_ROWS = 1024     # from here on a product that feeds the residual stream adds into it in the library
     MOE_ROUTE_FUSED_MAX_TOKENS = 0   # up to here one kernel computes router logits and choice; above, product + choice
     MOE_PAIRWISE_MAX_TOKENS = 2     # up to here a bfloat16 step's experts run pair by pair; above, grouped by expert
+    MFMA_ATTENTION_EXTRAS = False   # whether the matrix-core attention takes a sink and a bias by distance
     name = "hip"
 
     def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
@@ -275,10 +288,124 @@ class HipOps:
                    "to_activation: a float32 tensor and an output of its shape")
         self._ok(self.lib.psamd_to_activation(self._stream(), src.data_ptr(), out.data_ptr(), _code(out.dtype), src.numel()))
 
-    def swiglu(self, gate_up, out) -> None:
+    def swiglu(self, gate_up, out, activation: str = "silu") -> None:
+        """out = act(gate) * up for [gate | up] rows; ``activation`` is the gate's: "silu", "relu" or "gelu_tanh"."""
         t, inter = out.shape
         self._need(gate_up.shape == (t, 2 * inter) and gate_up.dtype == out.dtype, "swiglu: shapes")
-        self._ok(self.lib.psamd_swiglu(self._stream(), gate_up.data_ptr(), out.data_ptr(), _code(out.dtype), t, inter))
+        self._ok(self.lib.psamd_swiglu(self._stream(), gate_up.data_ptr(), out.data_ptr(), _code(out.dtype), t, inter,
+                                       GATE_ACTIVATIONS[activation]))
+
+    def residual_add(self, residual, delta) -> None:
+        """residual (float32 [T, H]) += delta: [T, H] in any kernel dtype, or [S, T, H] float32 slices
+        (added in ascending order). For an arrangement that adds a sub-layer's output without a
+        norm behind the sum."""
+        t, h = residual.shape
+        self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual_add: the stream is float32")
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, delta.dtype)
+        self._ok(self.lib.psamd_residual_add(self._stream(), residual.data_ptr(), dptr, dcode, slices, stride, t, h))
+
+    def stream_affine(self, x, factor: float = 1.0, row=None) -> None:
+        """x (float32 [T, H]) <- x * factor + row (float32 [H] or None), in place."""
+        t, h = x.shape
+        self._need(x.dtype == torch.float32 and x.is_contiguous(), "stream_affine: a float32 tensor")
+        if row is not None:
+            self._need(row.dtype == torch.float32 and row.numel() == h and row.is_contiguous(), "stream_affine: the row is float32 [H]")
+        self._ok(self.lib.psamd_stream_affine(self._stream(), x.data_ptr(), t, h, float(factor), _ptr(row)))
+
+    def concat_to_activation(self, a, b, out) -> None:
+        """out[t] = [a[t], b[t]] in out's dtype; a and b float32 [T, H]."""
+        t, h = a.shape
+        self._need(a.dtype == torch.float32 and b.dtype == torch.float32 and a.shape == b.shape and a.is_contiguous()
+                   and b.is_contiguous() and out.shape == (t, 2 * h) and out.is_contiguous(), "concat_to_activation: shapes")
+        self._ok(self.lib.psamd_concat_to_activation(self._stream(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                     _code(out.dtype), t, h))
+
+    def heads_linear(self, x, x_offset: int, x_head: int, w, out, out_offset: int, out_head: int) -> None:
+        """One small product per head: out[t, out_offset + h * out_head + n] = sum_k x[t, x_offset + h * x_head + k]
+        * w[h, n, k] for w [H, N, K]; x and out are 2-d and contiguous, their heads lie inside their
+        rows. One dtype for x, w and out; float accumulation."""
+        heads, n, k = w.shape
+        m = x.shape[0]
+        self._need(x.dim() == 2 and out.dim() == 2 and x.is_contiguous() and out.is_contiguous() and w.is_contiguous()
+                   and out.shape[0] == m, "heads_linear: operands")
+        self._need(x.dtype == w.dtype == out.dtype, "heads_linear: one dtype")
+        self._need(x_offset >= 0 and x_offset + (heads - 1) * x_head + k <= x.shape[1]
+                   and out_offset >= 0 and out_offset + (heads - 1) * out_head + n <= out.shape[1], "heads_linear: heads outside their rows")
+        size = x.element_size()
+        self._ok(self.lib.psamd_heads_linear(
+            self._stream(), x.data_ptr() + x_offset * size, _code(x.dtype), x.shape[1], x_head, w.data_ptr(), _code(w.dtype),
+            out.data_ptr() + out_offset * size, _code(out.dtype), out.shape[1], out_head, m, heads, n, k))
+
+    def latent_kv_append(self, rows, q_lat, hq: int, dim: int, rot: int, rank: int, slots: int, positions, table,
+                         norm_weight, eps: float, kv, write_slot) -> None:
+        """Latent attention between its input product and the attention: ``rows`` [T, hq (dim + rot) + rank + rot]
+        holds the heads' queries and the token's compressed vector with the shared key part. The
+        compressed vector is normalized (weight, eps), the key part and every head's last ``rot``
+        query dimensions are rotated pair by pair (neighbours; ``table`` [pos, rot/2, 2]); the page
+        receives key and value, ``q_lat`` [T, hq * slots] every head's rotated part at [rank, rank + rot)
+        and zeros behind it."""
+        t = rows.shape[0]
+        self._need(rows.is_contiguous() and q_lat.is_contiguous() and q_lat.dtype == rows.dtype
+                   and rows.shape[1] >= hq * (dim + rot) + rank + rot and q_lat.shape == (t, hq * slots), "latent_kv_append: shapes")
+        self._need(positions.dtype == torch.int32 and positions.numel() == t, "latent_kv_append: positions")
+        self._need(norm_weight.dtype == torch.float32 and norm_weight.numel() == rank and norm_weight.is_contiguous(),
+                   "latent_kv_append: the norm's weight is float32 [rank]")
+        if rot:
+            self._need(table is not None and table.dtype == torch.float32 and table.shape[1:] == (rot // 2, 2)
+                       and table.is_contiguous() and table.shape[0] >= 1, "latent_kv_append: table must be float32 [positions, rot/2, 2]")
+        if kv is not None:
+            self._need(kv.dtype == rows.dtype and kv.shape[1:] == (2, 1, 16 * slots) and kv.is_contiguous(),
+                       "latent_kv_append: cache must be [blocks, 2, 1, 16 * slots] in the activation dtype")
+            self._need(write_slot.dtype == torch.int32 and write_slot.numel() == t, "latent_kv_append: write slots")
+        self._ok(self.lib.psamd_latent_kv_append(self._stream(), rows.data_ptr(), rows.shape[1], q_lat.data_ptr(), _code(rows.dtype),
+                                                 t, hq, dim, rot, rank, slots, positions.data_ptr(), _ptr(table),
+                                                 norm_weight.data_ptr(), float(eps), _ptr(kv),
+                                                 None if kv is None else write_slot.data_ptr()))
+
+    def _state_args(self, state, ctx, width: int, taps: int) -> tuple:
+        self._need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+                   and state.shape[1] >= taps * width, "recurrence: the state is float32 [slots, taps * width]")
+        # Slot numbers are checked by the step packer against the number of slots the runner made.
+        return state.data_ptr(), state.shape[1]
+
+    def causal_conv(self, rows, col: int, bias, conv_w, conv_b, u, state, ctx) -> None:
+        """u[t, c] = conv_b[c] + sum_j conv_w[c, j] v(t - (taps - 1) + j, c), v = rows[:, col + c] + bias[c] over
+        each item's tokens, continued in front of the item's first token from the inputs its state
+        slot saved (``state`` [slots, taps * width]: taps - 1 saved inputs, oldest first, then the
+        recurrence's own row). ``u`` is float32 [T, width]. The state is only read."""
+        t, width = u.shape
+        taps = conv_w.shape[1]
+        self._need(rows.is_contiguous() and 0 <= col and col + width <= rows.shape[1] and rows.shape[0] == t, "causal_conv: rows")
+        self._need(u.dtype == torch.float32 and u.is_contiguous(), "causal_conv: u is float32")
+        for v, shape in ((bias, (width,)), (conv_w, (width, taps)), (conv_b, (width,))):
+            self._need(v.dtype == torch.float32 and tuple(v.shape) == shape and v.is_contiguous(), "causal_conv: float32 parameters")
+        self._need(t == ctx.num_tokens, "causal_conv: token count differs from the step batch")
+        sptr, srow = self._state_args(state, ctx, width, taps)
+        self._ok(self.lib.psamd_causal_conv(self._stream(), rows.data_ptr() + col * rows.element_size(), _code(rows.dtype),
+                                            rows.shape[1], bias.data_ptr(), conv_w.data_ptr(), conv_b.data_ptr(), u.data_ptr(),
+                                            sptr, srow, ctx.tok_item.data_ptr(), ctx.item_start.data_ptr(),
+                                            ctx.slots.data_ptr(), t, width, taps))
+
+    def gated_scan(self, gates, gate_bias, u, decay, rows, y_col: int, x_col: int, y_bias, x_bias, out, state, ctx,
+                   blocks: int, taps: int) -> None:
+        """The gated linear recurrence over each item's tokens from its state slot (see ``causal_conv`` for
+        the slot's layout): r, i = sigmoid(gates[t, b, :bw] + ., gates[t, b, bw:] + .), log a = decay * r,
+        S <- a S + sqrt(1 - a^2) i u; out = S * gelu_tanh(rows[:, y_col + c] + y_bias). Leaves S and the
+        item's last taps - 1 inputs (rows[:, x_col + c] + x_bias) in the slot."""
+        t, width = u.shape
+        self._need(gates.dtype == torch.float32 and gates.shape == (t, 2 * width) and gates.is_contiguous()
+                   and u.dtype == torch.float32 and u.is_contiguous(), "gated_scan: gates and u are float32")
+        self._need(width % blocks == 0 and out.shape == (t, width) and out.is_contiguous() and out.dtype == rows.dtype
+                   and rows.is_contiguous() and max(y_col, x_col) + width <= rows.shape[1] and rows.shape[0] == t, "gated_scan: shapes")
+        for v, n in ((gate_bias, 2 * width), (decay, width), (y_bias, width), (x_bias, width)):
+            self._need(v.dtype == torch.float32 and v.numel() == n and v.is_contiguous(), "gated_scan: float32 parameters")
+        self._need(t == ctx.num_tokens, "gated_scan: token count differs from the step batch")
+        sptr, srow = self._state_args(state, ctx, width, taps)
+        size = rows.element_size()
+        self._ok(self.lib.psamd_gated_scan(self._stream(), gates.data_ptr(), gate_bias.data_ptr(), u.data_ptr(), decay.data_ptr(),
+                                           rows.data_ptr() + y_col * size, rows.data_ptr() + x_col * size, _code(rows.dtype),
+                                           rows.shape[1], y_bias.data_ptr(), x_bias.data_ptr(), out.data_ptr(), sptr, srow,
+                                           ctx.item_start.data_ptr(), ctx.slots.data_ptr(), ctx.num_items, width, blocks, taps))
 
     def rope_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot) -> None:
         t = qkv.shape[0]
@@ -296,11 +423,36 @@ class HipOps:
                                                None if kv is None else write_slot.data_ptr()))
 
     def rope_norm_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot, norm_dim: int,
-                            norm_eps: float) -> None:
+                            norm_eps: float, bias=None, q_weight=None, k_weight=None, values_from_keys: bool = False) -> None:
         """``rope_kv_append`` with every q and k head divided, behind the rotation, by the root mean
         square over its ``norm_dim`` own dimensions (0: no norm; the head's other slots hold zeros).
-        ``hkv`` may be 0: rows of queries alone, nothing written to pages."""
+        ``hkv`` may be 0: rows of queries alone, nothing written to pages. ``bias`` (float32
+        [(hq + hkv) * d]) is added to the q and k heads first; ``q_weight`` / ``k_weight`` (float32 [d])
+        multiply the normalized heads; ``values_from_keys``: the rows are [q | k] only and the value
+        written to the pages is the key as projected (with its bias, before rotation and norm)."""
         t = qkv.shape[0]
+        general = bias is not None or q_weight is not None or k_weight is not None or values_from_keys
+        if general:
+            row_heads = hq + (hkv if values_from_keys else 2 * hkv)
+            self._need(qkv.shape[1] == row_heads * d and qkv.is_contiguous(), "rope_norm_kv_append: qkv shape")
+            self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_norm_kv_append: positions")
+            self._need(0 <= norm_dim <= d and d % 2 == 0 and d <= 256, "rope_norm_kv_append: head sizes")
+            for v, n in ((bias, (hq + hkv) * d), (q_weight, d), (k_weight, d)):
+                if v is not None:
+                    self._need(v.dtype == torch.float32 and v.numel() == n and v.is_contiguous(),
+                               "rope_norm_kv_append: bias and norm weights are float32")
+            if table is not None:
+                self._need(table.dtype == torch.float32 and table.shape[1:] == (d // 2, 2) and table.is_contiguous()
+                           and table.shape[0] >= 1, "rope_norm_kv_append: table must be float32 [positions, D/2, 2]")
+            if kv is not None:
+                self._need(hkv > 0 and kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                           "rope_norm_kv_append: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+                self._need(write_slot.dtype == torch.int32 and write_slot.numel() == t, "rope_norm_kv_append: write slots")
+            self._ok(self.lib.psamd_qk_prepare_kv_append(
+                self._stream(), qkv.data_ptr(), _code(qkv.dtype), t, hq, hkv, d, positions.data_ptr(), _ptr(table),
+                int(norm_dim), float(norm_eps), _ptr(bias), _ptr(q_weight), _ptr(k_weight), int(values_from_keys), _ptr(kv),
+                None if kv is None else write_slot.data_ptr()))
+            return
         self._need(qkv.shape[1] == (hq + 2 * hkv) * d and qkv.is_contiguous(), "rope_norm_kv_append: qkv shape")
         self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_norm_kv_append: positions")
         self._need(0 <= norm_dim <= d and d % 2 == 0 and d <= 256, "rope_norm_kv_append: head sizes")
@@ -440,7 +592,9 @@ class HipOps:
         self.linear(x, w, out)
         return out
 
-    def linear_swiglu(self, x, w_gate_up, out) -> None:
+    def linear_swiglu(self, x, w_gate_up, out, activation: str = "silu") -> None:
+        """out = act(x gate^T) * (x up^T) for w_gate_up = [gate; up]; ``activation`` is the gate's."""
+        epi = 1 + GATE_ACTIVATIONS[activation]       # the fused kernels' epilogue code
         m, k = x.shape
         inter = out.shape[1]
         self._need(w_gate_up.shape == (2 * inter, k) and out.shape[0] == m, "linear_swiglu: shapes")
@@ -451,7 +605,7 @@ class HipOps:
                 resid, rows, nw, nw_code, eps = self._normed_args(x, k)
                 self._need(w_gate_up.is_contiguous() and out.is_contiguous(), "linear_swiglu: operands")
                 self._ok(self.lib.psamd_linear_normed(self._stream(), resid, rows, nw, nw_code, eps, w_gate_up.data_ptr(),
-                                                      out.data_ptr(), _BF16, m, inter, k, 1))
+                                                      out.data_ptr(), _BF16, m, inter, k, epi))
                 return
             x = self.normed(x)
         self._need(x.is_contiguous() and w_gate_up.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
@@ -464,15 +618,15 @@ class HipOps:
                                         m, 2 * inter, k, 0 if self.fixed_kv_len else 1, 0)
             if rc != 2:                          # 2: no algorithm for this shape: the fused form below
                 self._ok(rc)
-                self.swiglu(gu, out)
+                self.swiglu(gu, out, activation)
                 return
         if small:
             self._ok(self.lib.psamd_linear_skinny(self._stream(), x.data_ptr(), w_gate_up.data_ptr(), out.data_ptr(),
-                                                  _BF16, m, inter, k, 1, 1))
+                                                  _BF16, m, inter, k, epi, 1))
             return
         gu = self.ws.get("mlp.gate_up", (m, 2 * inter), x.dtype)
         self.linear(x, w_gate_up, gu)
-        self.swiglu(gu, out)
+        self.swiglu(gu, out, activation)
 
     # ------------------------------------------------------------------ experts
 
@@ -575,10 +729,18 @@ class HipOps:
         return bool(self.lib.psamd_attention_mfma_supports(hq, hkv, d))
 
     def paged_attention(self, qkv, out, kv, ctx, group: int, hq: int, hkv: int, d: int, scale: float,
-                        window: int | None, exact_weights: bool = False) -> None:
+                        window: int | None, exact_weights: bool = False, sink=None, dist_bias=None) -> None:
         """``exact_weights``: the softmax weights enter the product with the values as computed in
         32-bit (the matrix-core kernels then take them as three bfloat16 terms that sum to the float32
-        weight exactly) instead of rounded to bfloat16; the 32-bit kernels always do."""
+        weight exactly) instead of rounded to bfloat16; the 32-bit kernels always do. ``sink``
+        (float32 [hq]): exp(sink) joins every softmax's denominator. ``dist_bias`` (float32 [hq, n]):
+        entry [h, min(i - j, n - 1)] is added to the scaled score of query i and key j."""
+        if sink is not None:
+            self._need(sink.dtype == torch.float32 and sink.numel() == hq and sink.is_contiguous(), "attention: sink is float32 [hq]")
+        if dist_bias is not None:
+            self._need(dist_bias.dtype == torch.float32 and dist_bias.dim() == 2 and dist_bias.shape[0] == hq
+                       and dist_bias.shape[1] >= 1 and dist_bias.is_contiguous(), "attention: distance bias is float32 [hq, n]")
+        extras = sink is not None or dist_bias is not None
         t = qkv.shape[0]
         g = ctx.groups[group]
         self._need(out.shape == (t, hq * d) and out.is_contiguous() and out.dtype == qkv.dtype, "attention: output")
@@ -588,7 +750,8 @@ class HipOps:
         win = int(window) if window is not None else 0
         stride = qkv.shape[1]
         s = self._stream()
-        if qkv.dtype == torch.bfloat16 and stride % 8 == 0 and self.mfma_attention_supported(hq, hkv, d):
+        if (qkv.dtype == torch.bfloat16 and stride % 8 == 0 and self.mfma_attention_supported(hq, hkv, d)
+                and (not extras or self.MFMA_ATTENTION_EXTRAS)):
             if ctx.num_prefill_tiles:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
                 # Few query tiles on a long context: the kernel deals their keys out to several
@@ -629,7 +792,8 @@ class HipOps:
             return
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),
-            ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win))
+            ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win,
+            _ptr(sink), _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1]))
 
     # ---------------------------------------------------------------- sampling
 

@@ -1,4 +1,5 @@
 """Architectures known to the registry. Importing this package registers them."""
 
+from . import gokolix  # noqa: F401
 from . import llama  # noqa: F401
 from . import radivik  # noqa: F401

@@ -51,6 +51,26 @@ def head_slots(head_dim: int, rotary_dim: int, slots: int) -> list[int]:
     return out
 
 
+def distance_bucket(n: int, buckets: int, far: float) -> int:
+    """The row of a learned bias table for a key ``n`` tokens back: the first half of the rows is one
+    row per distance; the other half covers the distances from there to ``far`` in steps that grow
+    geometrically; every distance from ``far`` on shares the last row."""
+    half = buckets // 2
+    if n < half:
+        return n
+    return min(buckets - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (buckets - half))))
+
+
+def distance_table(rel: torch.Tensor, far: float) -> torch.Tensor:
+    """[buckets, heads] -> float32 [heads, n]: the bias for every distance 0 .. n - 1, where the last
+    entry stands for every larger distance too (n - 1 >= far, so it reads the last row)."""
+    buckets = rel.shape[0]
+    n = max(int(math.ceil(far)), buckets // 2) + 1
+    rows = torch.tensor([distance_bucket(d, buckets, far) for d in range(n)], dtype=torch.long)
+    assert int(rows[-1]) == buckets - 1
+    return rel.to(torch.float32)[rows].t().contiguous()
+
+
 class PagedAttention(Mixer):
     """q/k/v projection (one fused product), position encoding on q and k, keys and values
     written to their pages, causal attention of every new token over the request's cache,
@@ -72,12 +92,23 @@ class PagedAttention(Mixer):
     * ``own_kv`` False: the layer has no key and value projections; its run reads the cache
       entry another run writes (``LayerRun.writes_cache`` False) with queries of its own.
     * ``exact_weights``: the softmax weights enter the product with the values as they were computed
-      in 32-bit instead of rounded to the activation dtype."""
+      in 32-bit instead of rounded to the activation dtype.
+    * ``qk_bias``: the q and k projections have biases (names "q_bias", "k_bias"), added in 32-bit.
+    * ``qk_norm_weights`` (with ``qk_norm_eps``): the normalized q and k heads are multiplied by
+      a weight of ``head_dim`` entries each, shared by the heads (names "q_norm", "k_norm").
+    * ``values_are_keys``: there is no value projection; a token's value is its key as
+      projected (with its bias, before rotation and norm).
+    * ``sink``: a learned number per head (name "sink") whose exponential joins the softmax's
+      denominator; it has no key and no value.
+    * ``distance_bias`` = {"buckets": B, "far": D}: a learned table [B, heads] (name "rel") whose
+      row bucket(i - j) is added to the scaled score of query i and key j (``distance_bucket``)."""
 
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], num_heads: int,
                  num_kv_heads: int, head_dim: int, names: Mapping[str, str], position: str | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
-                 qk_norm_eps: float | None = None, own_kv: bool = True, exact_weights: bool = False) -> None:
+                 qk_norm_eps: float | None = None, own_kv: bool = True, exact_weights: bool = False,
+                 qk_bias: bool = False, qk_norm_weights: bool = False, values_are_keys: bool = False,
+                 sink: bool = False, distance_bias: Mapping[str, Any] | None = None) -> None:
         if num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads not divisible by {num_kv_heads} kv heads")
         self.hidden_size = int(hidden_size)
@@ -86,6 +117,20 @@ class PagedAttention(Mixer):
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.own_kv = bool(own_kv)
         self.exact_weights = bool(exact_weights)
+        self.qk_bias, self.qk_norm_weights = bool(qk_bias), bool(qk_norm_weights)
+        self.values_are_keys, self.has_sink = bool(values_are_keys), bool(sink)
+        self.distance_bias = None if distance_bias is None else (int(distance_bias["buckets"]), float(distance_bias["far"]))
+        if self.qk_norm_weights and self.qk_norm_eps is None:
+            raise ValueError("weights on the q/k norm need qk_norm_eps")
+        if self.values_are_keys and (self.value_dim != self.head_dim or not self.own_kv):
+            raise ValueError("values that are the keys have the keys' size and belong to a layer with keys of its own")
+        if (self.qk_bias or self.qk_norm_weights) and not self.own_kv:
+            raise ValueError("biases and norm weights on q and k are implemented for layers with keys of their own")
+        if self.distance_bias is not None and not 2 <= self.distance_bias[0] < 2 * self.distance_bias[1]:
+            raise ValueError(f"a distance bias needs at least 2 buckets and a reach beyond half of them, got {self.distance_bias}")
+        extras = (self.qk_bias or self.qk_norm_weights or self.values_are_keys or self.has_sink
+                  or self.distance_bias is not None)
+        self.bias = self.q_norm_weight = self.k_norm_weight = self.sink = self.distance_table = None
         self.names = dict(names)
         self.window = None if window is None else int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
@@ -94,7 +139,7 @@ class PagedAttention(Mixer):
             raise ValueError("PagedAttention applies rotation tables; other encodings belong to their own mixer")
         rotary = self.head_dim if self.pos is None or self.pos.rotary_dim is None else int(self.pos.rotary_dim)
         self.plain = (self.value_dim == self.head_dim and rotary == self.head_dim and self.qk_norm_eps is None
-                      and self.own_kv)
+                      and self.own_kv and not extras)
         if self.plain:
             if head_dim % 16 or not 16 <= head_dim <= 256:
                 raise ValueError(f"head_dim must be a multiple of 16 in [16, 256], got {head_dim}")
@@ -111,6 +156,7 @@ class PagedAttention(Mixer):
         self.takes_normed_rows = self.plain
         self.q_size = self.num_heads * self.slots
         self.kv_size = self.num_kv_heads * self.slots if self.own_kv else 0
+        self.row_width = self.q_size + (1 if self.values_are_keys else 2) * self.kv_size
 
     def weights(self) -> dict[str, WeightWant]:
         h, n = self.hidden_size, self.names
@@ -118,7 +164,18 @@ class PagedAttention(Mixer):
                 n["o"]: WeightWant((h, self.num_heads * self.value_dim))}
         if self.own_kv:
             want[n["k"]] = WeightWant((self.num_kv_heads * self.head_dim, h))
-            want[n["v"]] = WeightWant((self.num_kv_heads * self.value_dim, h))
+            if not self.values_are_keys:
+                want[n["v"]] = WeightWant((self.num_kv_heads * self.value_dim, h))
+        if self.qk_bias:
+            want[n["q_bias"]] = WeightWant((self.num_heads * self.head_dim,), "bias")
+            want[n["k_bias"]] = WeightWant((self.num_kv_heads * self.head_dim,), "bias")
+        if self.qk_norm_weights:
+            want[n["q_norm"]] = WeightWant((self.head_dim,), "norm")
+            want[n["k_norm"]] = WeightWant((self.head_dim,), "norm")
+        if self.has_sink:
+            want[n["sink"]] = WeightWant((self.num_heads,), "bias")
+        if self.distance_bias is not None:
+            want[n["rel"]] = WeightWant((self.distance_bias[0], self.num_heads), "bias")
         return want
 
     def cache_need(self) -> CacheNeed:
@@ -143,12 +200,31 @@ class PagedAttention(Mixer):
         rows = [self._spread(tensors[n["q"]], self.num_heads, self.head_dim, self.index)]
         if self.own_kv:
             rows.append(self._spread(tensors[n["k"]], self.num_kv_heads, self.head_dim, self.index))
-            rows.append(self._spread(tensors[n["v"]], self.num_kv_heads, self.value_dim, None))
+            if not self.values_are_keys:
+                rows.append(self._spread(tensors[n["v"]], self.num_kv_heads, self.value_dim, None))
         self.w_qkv = rt.ops.prepare_matrix(torch.cat(rows, dim=0), rt)
         o = tensors[n["o"]]
         wide = torch.zeros((o.shape[0], self.num_heads, self.slots), dtype=o.dtype)
-        wide[:, :, : self.value_dim] = o.view(o.shape[0], self.num_heads, self.value_dim)
+        # A value that is the key lies in the key's slots.
+        cols = self.index if self.values_are_keys else list(range(self.value_dim))
+        wide[:, :, cols] = o.view(o.shape[0], self.num_heads, self.value_dim)
         self.w_o = rt.ops.prepare_matrix(wide.view(o.shape[0], self.num_heads * self.slots), rt)
+
+        def on_device(t: torch.Tensor) -> torch.Tensor:
+            return t.to(device=rt.device, dtype=torch.float32).contiguous()
+
+        self.bias = self.q_norm_weight = self.k_norm_weight = self.sink = self.distance_table = None
+        if self.qk_bias:
+            both = [self._spread(tensors[n[key]].to(torch.float32)[:, None], heads, self.head_dim, self.index)
+                    for key, heads in (("q_bias", self.num_heads), ("k_bias", self.num_kv_heads))]
+            self.bias = on_device(torch.cat(both, dim=0).view(-1))
+        if self.qk_norm_weights:
+            self.q_norm_weight = on_device(self._spread(tensors[n["q_norm"]].to(torch.float32)[:, None], 1, self.head_dim, self.index).view(-1))
+            self.k_norm_weight = on_device(self._spread(tensors[n["k_norm"]].to(torch.float32)[:, None], 1, self.head_dim, self.index).view(-1))
+        if self.has_sink:
+            self.sink = on_device(tensors[n["sink"]])
+        if self.distance_bias is not None:
+            self.distance_table = on_device(distance_table(tensors[n["rel"]].to(torch.float32), self.distance_bias[1]))
 
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
@@ -169,13 +245,24 @@ class PagedAttention(Mixer):
             # the pages (the statistic needs a whole head, which the fused product spreads over
             # workgroups).
             own = self.num_kv_heads if self.own_kv else 0
-            qkv = ws.get("attn.qkv" if own else "attn.q", (t, self.q_size + 2 * self.kv_size), rt.dtype)
+            qkv = ws.get("attn.qkv" if own else "attn.q", (t, self.row_width), rt.dtype)
             ops.linear(x, self.w_qkv, qkv)
-            ops.rope_norm_kv_append(qkv, self.num_heads, own, self.slots, ctx.positions, table,
-                                    cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
-                                    self.head_dim if self.qk_norm_eps is not None else 0, self.qk_norm_eps or 0.0)
+            norm_dim, eps = (self.head_dim, self.qk_norm_eps) if self.qk_norm_eps is not None else (0, 0.0)
+            if self.qk_bias or self.qk_norm_weights or self.values_are_keys:
+                ops.rope_norm_kv_append(qkv, self.num_heads, own, self.slots, ctx.positions, table,
+                                        cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
+                                        norm_dim, eps, bias=self.bias, q_weight=self.q_norm_weight,
+                                        k_weight=self.k_norm_weight, values_from_keys=self.values_are_keys)
+            else:
+                ops.rope_norm_kv_append(qkv, self.num_heads, own, self.slots, ctx.positions, table,
+                                        cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
+                                        norm_dim, eps)
         out = ws.get("attn.out", (t, self.q_size), rt.dtype)
-        if self.exact_weights:
+        if self.sink is not None or self.distance_table is not None:
+            ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
+                                self.slots, self.scale, cache.window, exact_weights=self.exact_weights,
+                                sink=self.sink, dist_bias=self.distance_table)
+        elif self.exact_weights:
             ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
                                 self.slots, self.scale, cache.window, exact_weights=True)
         else:

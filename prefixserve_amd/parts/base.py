@@ -23,7 +23,9 @@ if TYPE_CHECKING:
 @dataclass(frozen=True)
 class WeightWant:
     """A weight a part asks for. ``init`` tells the random-weights mode how to fill it:
-    "matrix" = N(0, std), "norm" = 1 + N(0, norm_std), "embedding" = N(0, std)."""
+    "matrix" = N(0, std), "norm" = 1 + N(0, norm_std), "embedding" = N(0, std), "offset" =
+    N(0, norm_std) (a norm weight stored as its distance from one), "bias" = N(0, 0.5) (biases,
+    sinks, small tables that are added to something of the order of one)."""
 
     shape: tuple[int, ...]
     init: str = "matrix"

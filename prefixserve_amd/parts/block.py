@@ -92,5 +92,35 @@ class PostNormBlock:
         return None
 
 
+class ParallelBlock:
+    """One norm, both sub-layers read it: x <- x + mixer(n(x)) + feed_forward(n(x)).
+
+    The normalized rows are written out by the norm kernel (never left to the consumers: the
+    mixer may add into the stream before the feed-forward has read it). The mixer's output goes
+    into the stream at once, the feed-forward's is handed on as ``pending`` for the next layer's
+    fused add+norm. ``feed_forward`` None: the layer is x <- x + mixer(n(x))."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm,
+                 feed_forward_norm: Norm | None = None) -> None:
+        if feed_forward_norm is not None:
+            raise ValueError("a parallel block has one norm")
+        self.mixer, self.feed_forward, self.mixer_norm = mixer, feed_forward, mixer_norm
+
+    def parts(self) -> list[Part]:
+        return [self.mixer_norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
+                state: torch.Tensor | None, writes_cache: bool) -> torch.Tensor | None:
+        ctx.stream_copy = None
+        h = self.mixer_norm.add_norm(residual, pending, "block.x")
+        mixed = self.mixer.forward(h, ctx, cache, state, writes_cache)
+        if self.feed_forward is None:
+            return mixed
+        if mixed is not None:
+            self.mixer_norm.rt.ops.residual_add(residual, mixed)
+        return self.feed_forward.forward(h, ctx)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("parallel", ParallelBlock)
 register_block("postnorm", PostNormBlock)

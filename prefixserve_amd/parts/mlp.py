@@ -13,16 +13,19 @@ if TYPE_CHECKING:
 
 
 class SwiGLU(FeedForward):
-    """down( silu(gate(x)) * up(x) ), no biases; gate and up are one fused product whose
+    """down( act(gate(x)) * up(x) ), no biases; gate and up are one fused product whose
     first ``intermediate_size`` columns are the gate (prefixserve/model/llama.py:120-121,
-    prefixserve/model/weights.py:120-123)."""
+    prefixserve/model/weights.py:120-123). ``activation`` is the gate's: "silu" (Llama), "relu"
+    or "gelu_tanh"."""
 
     takes_normed_rows = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str],
                  activation: str = "silu") -> None:
-        if activation != "silu":
-            raise ValueError(f"the gated feed-forward kernels apply SiLU to the gate; {activation!r} is not implemented")
+        if activation not in ("silu", "relu", "gelu_tanh"):
+            raise ValueError(f"the gated feed-forward kernels apply SiLU, ReLU or GELU (tanh form) to the gate; "
+                             f"{activation!r} is not implemented")
+        self.activation = activation
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.names = dict(names)
@@ -44,7 +47,10 @@ class SwiGLU(FeedForward):
         rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace
         t = x.shape[0]
         act = ws.get("mlp.act", (t, self.intermediate_size), rt.dtype)
-        ops.linear_swiglu(x, self.w_gate_up, act)
+        if self.activation == "silu":
+            ops.linear_swiglu(x, self.w_gate_up, act)
+        else:
+            ops.linear_swiglu(x, self.w_gate_up, act, activation=self.activation)
         return ops.linear_to_residual(act, self.w_down, "mlp.delta", getattr(ctx, "residual", None))
 
 

@@ -10,10 +10,13 @@ import torch
 
 from . import attention as _attention  # noqa: F401  (registers the built-in parts)
 from . import block as _block  # noqa: F401
+from . import latent as _latent  # noqa: F401
 from . import mlp as _mlp  # noqa: F401
 from . import moe as _moe  # noqa: F401
 from . import norm as _norm  # noqa: F401
+from . import recurrent as _recurrent  # noqa: F401
 from . import rope as _rope  # noqa: F401
+from . import stream as _stream  # noqa: F401
 from .base import CacheNeed, Part, Runtime, StateNeed, WeightWant, make
 from .spec import ModelSpec
 
@@ -43,6 +46,11 @@ class DecoderModel:
         sizes = dict(hidden_size=spec.hidden_size, vocab_size=spec.vocab_size)
         self.embedding_transforms = [make("transform", ps.kind, **sizes, **ps.params) for ps in spec.embedding_transforms]
         self.logit_transforms = [make("transform", ps.kind, **sizes, **ps.params) for ps in spec.logit_transforms]
+        self.stream_transforms = {name: make("transform", ps.kind, **sizes, **ps.params)
+                                  for name, ps in spec.stream_transforms.items()}
+        # The token table's output (behind its transforms) is kept for the step if a transform asks.
+        self.keeps_embedding_output = any(getattr(tr, "needs_embedding_output", False)
+                                          for tr in self.stream_transforms.values())
         self.caches: dict[int, Any] = {}
         self.states: dict[int, torch.Tensor] = {}
         self.rt: Runtime | None = None
@@ -54,7 +62,7 @@ class DecoderModel:
         for layer, blk in zip(self.spec.layers, self.blocks):
             out += [(layer.prefix, p) for p in blk.parts()]
         out.append((self.spec.final_norm_prefix, self.final_norm))
-        out += [("", tr) for tr in self.embedding_transforms + self.logit_transforms]
+        out += [("", tr) for tr in self.embedding_transforms + self.logit_transforms + list(self.stream_transforms.values())]
         return out
 
     def weights(self) -> dict[str, WeightWant]:
@@ -139,8 +147,21 @@ class DecoderModel:
                 tr.apply(residual, ctx, None)
             ctx.residual = residual
             ctx.stream_copy = None           # a context may be stepped twice (a graph's eager run, then its capture)
+            if self.keeps_embedding_output:
+                ctx.embedding_output = ws.get("embedding.output", (t, s.hidden_size), torch.float32)
+                ctx.embedding_output.copy_(residual)
             pending = None
             for i, run in enumerate(s.order):
+                if run.before:
+                    # A transform reads and writes the stream itself: what the last sub-layer left to
+                    # be added goes in first.
+                    if pending is not None:
+                        ops.residual_add(residual, pending)
+                        pending = None
+                    ctx.stream_copy = None
+                    ctx.pass_index = run.pass_index
+                    for name in run.before:
+                        self.stream_transforms[name].apply(residual, ctx, None)
                 pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),
                                                          self.states.get(i), run.writes_cache)
             if ctx.num_logit_rows == 0:

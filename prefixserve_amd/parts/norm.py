@@ -12,21 +12,26 @@ from .base import Norm, NormedRows, Runtime, WeightWant, register_norm
 class RMSNorm(Norm):
     """weight * x * rsqrt(mean(x^2) + eps), eps inside the root; statistics, scale and the
     residual sum in 32-bit (prefixserve/model/llama.py:63-69 of the reference upcasts the
-    same way). The weight is used in the dtype it is stored in."""
+    same way). The weight is used in the dtype it is stored in. ``unit_offset``: the stored
+    tensor is the weight's distance from one, the factor is 1 + w (formed in 32-bit and kept so:
+    rounding 1 + w to the stored 16 bits would drop most of w)."""
 
-    def __init__(self, hidden_size: int, eps: float, name: str = "weight") -> None:
+    def __init__(self, hidden_size: int, eps: float, name: str = "weight", unit_offset: bool = False) -> None:
         self.hidden_size = int(hidden_size)
         self.eps = float(eps)
         self.name = name
+        self.unit_offset = bool(unit_offset)
 
     def weights(self) -> dict[str, WeightWant]:
-        return {self.name: WeightWant((self.hidden_size,), "norm")}
+        return {self.name: WeightWant((self.hidden_size,), "offset" if self.unit_offset else "norm")}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         super().bind(tensors, rt)
         w = tensors[self.name]
         if w.dtype not in (torch.bfloat16, torch.float32):
             w = w.to(torch.float32)
+        if self.unit_offset:
+            w = 1.0 + w.to(torch.float32)
         self.weight = w.to(rt.device).contiguous()
 
     def weight_bytes(self) -> int:

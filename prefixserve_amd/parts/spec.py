@@ -46,11 +46,17 @@ class LayerRun:
     the others only read it, which is how a layer reads another layer's keys and values.
     A layer may appear in several runs (the same weights applied twice); each run that
     writes needs a cache entry of its own.
+
+    ``before`` names transforms of the residual stream (``ModelSpec.stream_transforms``) that are
+    applied in front of this run, in that order; ``pass_index`` says which time through a
+    repeated stretch of layers the run belongs to, for transforms that differ from pass to pass.
     """
 
     layer: int
     cache: int
     writes_cache: bool = True
+    before: tuple[str, ...] = ()
+    pass_index: int = 0
 
 
 @dataclass(frozen=True)
@@ -72,12 +78,18 @@ class ModelSpec:
     # weight names are taken as they are, without a prefix.
     embedding_transforms: tuple[PartSpec, ...] = ()
     logit_transforms: tuple[PartSpec, ...] = ()
+    # Named transforms of the residual stream between layers (a re-entry into a repeated stretch,
+    # say), applied where a ``LayerRun.before`` names them; each is built once.
+    stream_transforms: Mapping[str, PartSpec] = field(default_factory=dict)
 
     def validate(self) -> None:
         writers: dict[int, int] = {}
         for run in self.order:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"order names layer {run.layer}, model has {len(self.layers)}")
+            for name in run.before:
+                if name not in self.stream_transforms:
+                    raise ValueError(f"a run names the stream transform {name!r}, which the model does not have")
             if run.writes_cache:
                 if run.cache in writers:
                     raise ValueError(f"cache entry {run.cache} is written by two runs")

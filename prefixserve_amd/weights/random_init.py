@@ -38,6 +38,10 @@ def random_tensors(wanted: Mapping[str, WeightWant], seed: int, std: float = 0.0
         t = torch.empty(want.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=g)
         if want.init == "norm":
             t = 1.0 + norm_std * t
+        elif want.init == "offset":              # a norm weight stored as its distance from one
+            t = norm_std * t
+        elif want.init == "bias":                # biases, sinks, small tables: of the order of one
+            t = 0.5 * t
         else:
             t = std * t
         out[name] = t.to(dtype).contiguous()

@@ -53,10 +53,97 @@ class EmulatedOps:
         self.linear(x, w, out)
         return out
 
-    def linear_swiglu(self, x, w_gate_up, out) -> None:
+    def linear_swiglu(self, x, w_gate_up, out, activation="silu") -> None:
         gu = x.float() @ w_gate_up.float().T
         inter = gu.shape[1] // 2
-        out.copy_((torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]).to(out.dtype))
+        act = {"silu": torch.nn.functional.silu, "relu": torch.relu,
+               "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh")}[activation]
+        out.copy_((act(gu[:, :inter]) * gu[:, inter:]).to(out.dtype))
+
+    def residual_add(self, residual, delta) -> None:
+        residual.add_(delta.float().sum(0) if delta.dim() == 3 else delta.float())
+
+    def stream_affine(self, x, factor=1.0, row=None) -> None:
+        x.mul_(factor)
+        if row is not None:
+            x.add_(row)
+
+    def concat_to_activation(self, a, b, out) -> None:
+        out.copy_(torch.cat([a, b], dim=-1).to(out.dtype))
+
+    def heads_linear(self, x, x_offset, x_head, w, out, out_offset, out_head) -> None:
+        heads, n, k = w.shape
+        for h in range(heads):
+            xs = x[:, x_offset + h * x_head: x_offset + h * x_head + k].float()
+            out[:, out_offset + h * out_head: out_offset + h * out_head + n] = (xs @ w[h].float().T).to(out.dtype)
+
+    def latent_kv_append(self, rows, q_lat, hq, dim, rot, rank, slots, positions, table, norm_weight, eps, kv, write_slot) -> None:
+        t = rows.shape[0]
+        low = rows[:, hq * (dim + rot):].float()
+        c = low[:, :rank]
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_weight
+
+        def turn(v):                                       # [..., rot], neighbours paired
+            cs = table[positions.long()]                   # [t, rot/2, 2]
+            while cs.dim() - 1 < v.dim():
+                cs = cs.unsqueeze(1)
+            a, b = v[..., 0::2], v[..., 1::2]
+            res = torch.empty_like(v)
+            res[..., 0::2] = a * cs[..., 0] - b * cs[..., 1]
+            res[..., 1::2] = b * cs[..., 0] + a * cs[..., 1]
+            return res
+
+        key = torch.zeros((t, slots))
+        key[:, :rank] = c
+        if rot:
+            key[:, rank: rank + rot] = turn(low[:, rank: rank + rot])
+        val = torch.zeros((t, slots))
+        val[:, :rank] = c
+        if kv is not None:
+            page, off = (write_slot // PAGE).long(), (write_slot % PAGE).long()
+            kv[:, 0].view(kv.shape[0], 1, PAGE, slots)[page, 0, off, :] = key.to(kv.dtype)
+            kv[:, 1].view(kv.shape[0], 1, slots, PAGE)[page, 0, :, off] = val.to(kv.dtype)
+        q = rows[:, : hq * (dim + rot)].view(t, hq, dim + rot).float()
+        ql = q_lat.view(t, hq, slots)
+        ql[:, :, rank:] = 0
+        if rot:
+            ql[:, :, rank: rank + rot] = turn(q[:, :, dim:]).to(q_lat.dtype)
+
+    def causal_conv(self, rows, col, bias, conv_w, conv_b, u, state, ctx) -> None:
+        width, taps = conv_w.shape
+        starts = ctx.item_start.tolist()
+        for i in range(ctx.num_items):
+            t0, t1 = starts[i], starts[i + 1]
+            slot = int(ctx.slots[i])
+            saved = state[slot, : (taps - 1) * width].view(taps - 1, width)
+            v = torch.cat([saved, rows[t0:t1, col: col + width].float() + bias], dim=0)
+            acc = conv_b.expand(t1 - t0, width).clone()
+            for j in range(taps):
+                acc += conv_w[:, j] * v[j: j + t1 - t0]
+            u[t0:t1] = acc
+
+    def gated_scan(self, gates, gate_bias, u, decay, rows, y_col, x_col, y_bias, x_bias, out, state, ctx, blocks, taps) -> None:
+        t, width = u.shape
+        bw = width // blocks
+        g = gates.view(t, blocks, 2 * bw) + gate_bias.view(blocks, 2 * bw)
+        r = torch.sigmoid(g[:, :, :bw]).reshape(t, width)
+        gi = torch.sigmoid(g[:, :, bw:]).reshape(t, width)
+        la = decay * r
+        a, step = torch.exp(la), torch.sqrt(-torch.expm1(2 * la))
+        y = torch.nn.functional.gelu(rows[:, y_col: y_col + width].float() + y_bias, approximate="tanh")
+        starts = ctx.item_start.tolist()
+        for i in range(ctx.num_items):
+            t0, t1 = starts[i], starts[i + 1]
+            slot = int(ctx.slots[i])
+            s = state[slot, (taps - 1) * width:].clone()
+            for k in range(t0, t1):
+                s = a[k] * s + step[k] * gi[k] * u[k]
+                out[k] = (s * y[k]).to(out.dtype)
+            state[slot, (taps - 1) * width:] = s
+            if taps > 1:
+                saved = state[slot, : (taps - 1) * width].view(taps - 1, width)
+                v = torch.cat([saved, rows[t0:t1, x_col: x_col + width].float() + x_bias], dim=0)
+                state[slot, : (taps - 1) * width] = v[-(taps - 1):].reshape(-1)
 
     def qkv_rope_append(self, x, w_qkv, qkv, hq, hkv, d, positions, table, kv, write_slot) -> None:
         self.linear(x, w_qkv, qkv)
@@ -97,10 +184,14 @@ class EmulatedOps:
         if out is not None:
             out.copy_(y.to(out.dtype))
 
-    def rope_norm_kv_append(self, qkv, hq, hkv, d, positions, table, kv, write_slot, norm_dim, norm_eps) -> None:
+    def rope_norm_kv_append(self, qkv, hq, hkv, d, positions, table, kv, write_slot, norm_dim, norm_eps, bias=None,
+                            q_weight=None, k_weight=None, values_from_keys=False) -> None:
         t = qkv.shape[0]
         heads = qkv[:, : (hq + hkv) * d].view(t, hq + hkv, d)
         x = heads.float()
+        if bias is not None:
+            x = x + bias.view(hq + hkv, d)
+        raw_keys = x[:, hq:].to(qkv.dtype)
         if table is not None:
             cs = table[positions.long()]
             cos, sin = cs[..., 0][:, None, :], cs[..., 1][:, None, :]
@@ -108,11 +199,16 @@ class EmulatedOps:
             x = torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
         if norm_dim:
             x = x * torch.rsqrt((x * x).sum(-1, keepdim=True) / norm_dim + norm_eps)
+        if q_weight is not None:
+            x[:, :hq] = x[:, :hq] * q_weight
+        if k_weight is not None:
+            x[:, hq:] = x[:, hq:] * k_weight
         heads.copy_(x.to(qkv.dtype))
         if kv is not None:
             page, off = (write_slot // PAGE).long(), (write_slot % PAGE).long()
             kv[:, 0].view(kv.shape[0], hkv, PAGE, d)[page, :, off, :] = heads[:, hq:]
-            kv[:, 1].view(kv.shape[0], hkv, d, PAGE)[page, :, :, off] = qkv[:, (hq + hkv) * d:].view(t, hkv, d)
+            vals = raw_keys if values_from_keys else qkv[:, (hq + hkv) * d:].view(t, hkv, d)
+            kv[:, 1].view(kv.shape[0], hkv, d, PAGE)[page, :, :, off] = vals
 
     def moe_route(self, x, w_router, chosen, weight, w_router_act=None) -> None:
         s = torch.sigmoid(x.float() @ w_router.float().T)
@@ -137,7 +233,8 @@ class EmulatedOps:
         """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
         return x.repeat_interleave(rep, dim=1)
 
-    def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window, exact_weights=False) -> None:
+    def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window, exact_weights=False, sink=None,
+                        dist_bias=None) -> None:
         g = ctx.groups[group]
         t = qkv.shape[0]
         q = qkv[:, : hq * d].view(t, hq, d).float()
@@ -160,8 +257,14 @@ class EmulatedOps:
             hidden = kpos > qpos
             if window is not None:
                 hidden = hidden | (qpos - kpos >= window)
+            if dist_bias is not None:
+                scores = scores + dist_bias[:, (qpos - kpos).clamp(0, dist_bias.shape[1] - 1)]
             scores = scores.masked_fill(hidden, float("-inf"))
+            if sink is not None:
+                scores = torch.cat([scores, sink.view(hq, 1, 1).expand(hq, scores.shape[1], 1)], dim=-1)
             probs = torch.softmax(scores, dim=-1)
+            if sink is not None:
+                probs = probs[..., :-1]
             o[t0:t1] = torch.matmul(probs, vals.transpose(0, 1)).transpose(0, 1).to(out.dtype)
 
     def argmax(self, logits, out) -> None:
