@@ -32,6 +32,11 @@ def plan_groups(needs: Mapping[int, CacheNeed]) -> list[LayerGroup]:
     by_need: dict[CacheNeed, list[int]] = {}
     for entry in sorted(needs):
         by_need.setdefault(needs[entry], []).append(entry)
+    if not by_need:
+        # A model none of whose mixers caches keys (recurrences alone): one group without entries,
+        # so that a request still has a block table and the scheduler its count of pages; its
+        # pages take no memory.
+        return [LayerGroup(CacheNeed(1, 16, None), ())]
     return [LayerGroup(need, tuple(entries)) for need, entries in by_need.items()]
 
 

@@ -159,7 +159,8 @@ class ModelRunner:
         torch.cuda.empty_cache()             # the throwaway pool goes back to the device; the step's buffers are in use
         free, _total = torch.cuda.mem_get_info(self.device)
         usable = free - reserve_bytes
-        n = int(usable // sum(self.bytes_per_block))
+        per_page = sum(self.bytes_per_block)
+        n = int(usable // per_page) if per_page else 4 * -(-self.max_seq_len // PAGE) * self.max_num_seqs
         n = min(n, (1 << 27) - 1)            # a token's place, page * 16 + offset, is a 32-bit integer
         need = -(-self.max_seq_len // PAGE)
         if n < need:
