@@ -213,6 +213,20 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
                            int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys,
                            int exact_weights);
 
+// psamd_attention_prefill and psamd_attention_decode with a sink and a bias by distance (see
+// psamd_attention_generic for both; either may be NULL).
+int psamd_attention_prefill_extras(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
+                                   const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks,
+                                   int max_kv_len, const int32_t* item_start, const int32_t* item_pos0,
+                                   const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
+                                   float scale, int window, float* part_o, float* part_ml, int nsplit, int exact_weights,
+                                   const float* sink, const float* dist_bias, int n_dist);
+int psamd_attention_decode_extras(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
+                                  float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+                                  const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
+                                  int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys,
+                                  int exact_weights, const float* sink, const float* dist_bias, int n_dist);
+
 // out[r] = argmax (temperature[r] <= 0) or the inverse-CDF draw with uniform[r] in [0, 1).
 int64_t psamd_sample_scratch_floats(int rows);
 int psamd_sample(void* stream, const float* logits, const float* temperature, const float* uniform, int32_t* out,

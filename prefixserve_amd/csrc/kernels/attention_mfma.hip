@@ -29,6 +29,18 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// What a softmax may have beyond keys: a learned sink per head (exp(sink[h]) joins the denominator;
+// it has no key and no value) and a bias on the scaled score that depends on the head and on how
+// far back the key lies, bias[h][min(i - j, n_dist - 1)]. Either pointer may be null. The entry
+// points with these arguments set g_extras for the launches they make.
+struct Extras {
+  const float* sink;
+  const float* bias;
+  int n_dist;
+};
+static thread_local Extras g_extras = {nullptr, nullptr, 0};
+constexpr float kLog2e = 1.44269504088896340736f;
 // A 16-byte piece in registers. A plain vector: HIP's uint4 is a struct, and copies of it in
 // arrays were compiled to copies through scratch memory.
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -105,7 +117,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, Extras ex) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int DTC = DT < 2 ? DT : 2;      // d-tiles merged per pass (bounds the LDS buffer)
@@ -216,6 +228,16 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     f32x16 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[0], qf[0], zero, 0, 0, 0);
 #pragma unroll
     for (int i = 1; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[i], qf[i], s, 0, 0, 0);
+    if (ex.bias != nullptr) {
+      // The bias is added to the scaled score: here the score is still unscaled.
+      const float* bt = ex.bias + static_cast<int64_t>(h) * ex.n_dist;
+      const float unscale = 1.f / scale;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+        s[v] = fmaf(bt[min(max(q_pos - key, 0), ex.n_dist - 1)], unscale, s[v]);
+      }
+    }
     // A tile whose last key is not after the first query, with no window, needs no mask.
     if (window > 0 || k0 + 31 > first_pos) {
 #pragma unroll
@@ -306,6 +328,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     if (w == wave) mine = f;
   }
   // One run of several: the sum, the maximum and the output as it is go to the merge kernel.
+  if (nsplit == 1 && ex.sink != nullptr) ll += __builtin_amdgcn_exp2f(ex.sink[h] * kLog2e - mm);   // one run: the sink joins here
   const float inv = nsplit > 1 ? 1.f : 1.f / ll;
   if (nsplit > 1 && wave == 0 && q_valid && hi == 0) {
     part_ml[2 * part_slot] = mm;
@@ -383,7 +406,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
     const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int n_tiles, int hq, int hkv, int table_pages, float scale,
     int window, float* __restrict__ part_o, float* __restrict__ part_ml, int pair_tiles, int tiles_per_wg,
-    const int32_t* __restrict__ pf_blocks, int n_blocks) {
+    const int32_t* __restrict__ pf_blocks, int n_blocks, Extras ex) {
   constexpr int D = 16 * NS;
   constexpr int DT = (D + 31) / 32;
   constexpr int KS = D + 8;                      // elements per key row in LDS
@@ -567,6 +590,17 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
       for (int i = 1; i < NS; ++i)
         s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ld8(kd + t * 32 * KS + 16 * i), qf[i], s[t], 0, 0, 0);
     }
+    if (ex.bias != nullptr) {
+      const float* bt = ex.bias + static_cast<int64_t>(h) * ex.n_dist;
+      const float unscale = 1.f / scale;
+#pragma unroll
+      for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * hi + (v & 3);
+          s[t][v] = fmaf(bt[min(max(q_pos - key, 0), ex.n_dist - 1)], unscale, s[t][v]);
+        }
+    }
     // Keys that are not after the first query, with no window, need no mask.
     if (window > 0 || k0 + 32 * KT - 1 > first_pos) {
 #pragma unroll
@@ -715,6 +749,7 @@ __global__ __launch_bounds__(256 * KP, NS <= 4 ? 4 : 2) void attn_prefill_groupe
       }
     return;
   }
+  if (ex.sink != nullptr) l += __builtin_amdgcn_exp2f(ex.sink[h] * kLog2e - m);
   const float inv = 1.f / l;
   bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
 #pragma unroll
@@ -745,7 +780,7 @@ constexpr int kMaxPrefillSplit = 16;
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
     const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ item_start, int64_t pairs, int hq, int d,
-    int nsplit) {
+    int nsplit, Extras ex) {
   const int per_pair = d >> 2;                         // threads per pair
   const int pairs_per_block = 256 / per_pair;
   const int sub = threadIdx.x / per_pair, chunk = threadIdx.x - sub * per_pair;
@@ -782,6 +817,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(
       acc.w += w * part[s].w;
     }
   }
+  if (ex.sink != nullptr) ll += __builtin_amdgcn_exp2f(ex.sink[h] * kLog2e - mm);
   const float inv = 1.f / ll;
   ushort4 pk;
   pk.x = float_to_bf16(acc.x * inv);
@@ -803,7 +839,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const int32_t* __restrict__ item_start,
     const int32_t* __restrict__ item_end, const int32_t* __restrict__ table_off,
     const int32_t* __restrict__ block_ids, int hq, int hkv, int nsplit, float scale, int window, int min_tiles,
-    int n_dec) {
+    int n_dec, Extras ex) {
   constexpr int D = 16 * NS;
   constexpr int KS = (D + 31) / 32;
   extern __shared__ float smem[];
@@ -925,11 +961,19 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       }
       float sv[8];
       float mx = -INFINITY;
+      // This lane's column of the tile is query head ct * 16 + r of the kv head's group.
+      const float* bt = ex.bias != nullptr
+                            ? ex.bias + static_cast<int64_t>(kvh * group + min(ct * 16 + r, group - 1)) * ex.n_dist : nullptr;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int key0 = k0 + 4 * g4 + v, key1 = key0 + 16;
-        sv[v] = (key0 <= pos && key0 >= k_lo) ? s0[v] * scale : -INFINITY;
-        sv[v + 4] = (key1 <= pos && key1 >= k_lo) ? s1[v] * scale : -INFINITY;
+        float b0 = 0.f, b1 = 0.f;
+        if (bt != nullptr) {
+          b0 = bt[min(max(pos - key0, 0), ex.n_dist - 1)];
+          b1 = bt[min(max(pos - key1, 0), ex.n_dist - 1)];
+        }
+        sv[v] = (key0 <= pos && key0 >= k_lo) ? fmaf(s0[v], scale, b0) : -INFINITY;
+        sv[v + 4] = (key1 <= pos && key1 >= k_lo) ? fmaf(s1[v], scale, b1) : -INFINITY;
         mx = fmaxf(mx, fmaxf(sv[v], sv[v + 4]));
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
@@ -998,6 +1042,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       ll += wgt * sm_l[w * group + hh];
     }
     if (nsplit == 1) {   // nothing to merge with: this is the result
+      if (ex.sink != nullptr) ll += __expf(ex.sink[kvh * group + hh] - mm);
       out[t * (static_cast<int64_t>(hq) * D) + static_cast<int64_t>(kvh * group + hh) * D + d] = float_to_bf16(acc / ll);
       continue;
     }
@@ -1016,7 +1061,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // not depend on each other.
 __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-    const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start, int hq, int d, int nsplit) {
+    const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start, int hq, int d, int nsplit, Extras ex) {
   __shared__ float wgt_s[64];
   const int di = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int64_t t = item_start[dec_items[di]];
@@ -1031,7 +1076,8 @@ __global__ __launch_bounds__(64) void attn_decode_merge_kernel(
   for (int s = 0; s < kEarly; ++s) early[s] = (s < nsplit && lane < d) ? part_o[(base + s) * d + lane] : 0.f;
   const float mm = wave_max(ms);
   const float w = ms == -INFINITY ? 0.f : __expf(ms - mm);
-  const float ll = wave_sum(w * ls);
+  float ll = wave_sum(w * ls);
+  if (ex.sink != nullptr) ll += __expf(ex.sink[h] - mm);
   wgt_s[lane] = w / ll;
   __syncthreads();
   for (int i = lane; i < d; i += kWave) {
@@ -1109,7 +1155,7 @@ static int launch_prefill_merge(hipStream_t s, const float* part_o, const float*
   const int64_t pairs = 32LL * n_tiles * hq;
   const int pairs_per_block = 256 / (head_dim / 4);
   attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(ceil_div(pairs, pairs_per_block))), dim3(256), 0, s>>>(
-      part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, pairs, hq, head_dim, nsplit);
+      part_o, part_ml, static_cast<bf16_t*>(out), pf_tiles, item_start, pairs, hq, head_dim, nsplit, g_extras);
   return check_launch("psamd_attention_prefill(merge)");
 }
 
@@ -1193,7 +1239,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
       attn_prefill_grouped_kernel<NS, 1, KP_, P3><<<grid, dim3(256 * KP_), smem, s>>>(                            \
           static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv),   \
           pf_tiles, item_start, item_pos0, table_off, block_ids, n_tiles, hq, hkv, table_pages, scale, window,   \
-          part_o, part_ml, pair, tiles_per_wg, pf_blocks, n_blocks);                                              \
+          part_o, part_ml, pair, tiles_per_wg, pf_blocks, n_blocks, g_extras);                                    \
       const int rc = check_launch("psamd_attention_prefill");                                                     \
       if (rc != 0 || nsplit == 1) return rc;                                                                      \
       return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);   \
@@ -1209,7 +1255,7 @@ static int launch_prefill(hipStream_t s, const void* qkv, int q_stride, void* ou
   }
   attn_prefill_mfma_kernel<NS, P3><<<dim3(hq, n_tiles, nsplit), dim3(256), sizeof(int32_t) * static_cast<size_t>(table_pages), s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), pf_tiles,
-      item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml);
+      item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, part_o, part_ml, g_extras);
   const int rc = check_launch("psamd_attention_prefill");
   if (rc != 0 || nsplit == 1) return rc;
   return launch_prefill_merge(s, part_o, part_ml, out, pf_tiles, item_start, n_tiles, hq, 16 * NS, nsplit);
@@ -1225,7 +1271,8 @@ static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const voi
   const int64_t groups_of_8 = ceil_div(static_cast<int64_t>(n_dec) * nsplit, 8);
   attn_decode_mfma_kernel<NS, CT, P3><<<dim3(8 * hkv, static_cast<unsigned>(groups_of_8)), dim3(256), smem, s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), static_cast<bf16_t*>(out), part_o,
-      part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles, n_dec);
+      part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles, n_dec,
+      g_extras);
   return check_launch("psamd_attention_decode");
 }
 
@@ -1406,8 +1453,39 @@ int psamd_attention_decode(void* stream, const void* qkv, int q_stride, void* ou
 #undef PSAMD_DEC_NS
   if (rc != 0 || nsplit == 1) return rc;
   attn_decode_merge_kernel<<<dim3(n_dec, hq), dim3(64), 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), dec_items,
-                                                               item_start, hq, head_dim, nsplit);
+                                                               item_start, hq, head_dim, nsplit, g_extras);
   return check_launch("psamd_attention_decode(merge)");
+}
+
+// The two entry points above with a softmax that has more than keys: sink (float [hq] or NULL) and
+// dist_bias (float [hq, n_dist] or NULL), see psamd_attention_generic.
+int psamd_attention_prefill_extras(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
+                                   const int32_t* pf_tiles, int n_tiles, const int32_t* pf_blocks, int n_blocks,
+                                   int max_kv_len, const int32_t* item_start, const int32_t* item_pos0,
+                                   const int32_t* table_off, const int32_t* block_ids, int hq, int hkv, int head_dim,
+                                   float scale, int window, float* part_o, float* part_ml, int nsplit, int exact_weights,
+                                   const float* sink, const float* dist_bias, int n_dist) {
+  PSAMD_REQUIRE(dist_bias == nullptr || (n_dist >= 1 && scale != 0.f), "a distance bias needs entries and a scale that is not zero");
+  g_extras = Extras{sink, dist_bias, n_dist};
+  const int rc = psamd_attention_prefill(stream, qkv, q_stride, out, kv, pf_tiles, n_tiles, pf_blocks, n_blocks, max_kv_len,
+                                         item_start, item_pos0, table_off, block_ids, hq, hkv, head_dim, scale, window,
+                                         part_o, part_ml, nsplit, exact_weights);
+  g_extras = Extras{nullptr, nullptr, 0};
+  return rc;
+}
+
+int psamd_attention_decode_extras(void* stream, const void* qkv, int q_stride, void* out, const void* kv, float* part_o,
+                                  float* part_ml, const int32_t* dec_items, int n_dec, const int32_t* item_start,
+                                  const int32_t* item_end, const int32_t* table_off, const int32_t* block_ids, int hq,
+                                  int hkv, int head_dim, int nsplit, float scale, int window, int min_split_keys,
+                                  int exact_weights, const float* sink, const float* dist_bias, int n_dist) {
+  PSAMD_REQUIRE(dist_bias == nullptr || n_dist >= 1, "a distance bias needs at least one entry per head");
+  g_extras = Extras{sink, dist_bias, n_dist};
+  const int rc = psamd_attention_decode(stream, qkv, q_stride, out, kv, part_o, part_ml, dec_items, n_dec, item_start,
+                                        item_end, table_off, block_ids, hq, hkv, head_dim, nsplit, scale, window,
+                                        min_split_keys, exact_weights);
+  g_extras = Extras{nullptr, nullptr, 0};
+  return rc;
 }
 
 }  // extern "C"

@@ -69,6 +69,10 @@ _SIGNATURES = {
                                 _f32, _i32, _vp, _vp, _i32, _i32],
     "psamd_attention_decode": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
                                _i32, _f32, _i32, _i32, _i32],
+    "psamd_attention_prefill_extras": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                                       _f32, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32],
+    "psamd_attention_decode_extras": [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                                      _i32, _f32, _i32, _i32, _i32, _vp, _vp, _i32],
     "psamd_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32],
     "psamd_scaled_add_rmsnorm": [_vp, _vp, _f32, _vp, _i32, _i32, _i64, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
@@ -100,7 +104,7 @@ class HipOps:
     LIBRARY_ADD_MIN_ROWS = 1024     # from here on a product that feeds the residual stream adds into it in the library
     MOE_ROUTE_FUSED_MAX_TOKENS = 0   # up to here one kernel computes router logits and choice; above, product + choice
     MOE_PAIRWISE_MAX_TOKENS = 2     # up to here a bfloat16 step's experts run pair by pair; above, grouped by expert
-    MFMA_ATTENTION_EXTRAS = False   # whether the matrix-core attention takes a sink and a bias by distance
+    MFMA_ATTENTION_EXTRAS = True    # whether the matrix-core attention takes a sink and a bias by distance
     name = "hip"
 
     def __init__(self, device: torch.device | str, workspace: Any = None) -> None:
@@ -766,13 +770,14 @@ class HipOps:
                 part_ml = self.ws.get("attn.prefill_part_ml", (rows * hq * 2,), torch.float32)
                 if nsplit > 1:
                     self._need(32 * ctx.num_prefill_tiles * nsplit <= rows, "attention: more split tiles than planned for")
-                self._ok(self.lib.psamd_attention_prefill(
+                tail = (_ptr(sink), _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1]) if extras else ()
+                self._ok((self.lib.psamd_attention_prefill_extras if extras else self.lib.psamd_attention_prefill)(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
                     ctx.num_prefill_tiles, ctx.pf_blocks.data_ptr(), ctx.num_prefill_blocks, kv_len,
                     ctx.item_start.data_ptr(), ctx.item_pos0.data_ptr(),
                     g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, scale, win,
                     part_o.data_ptr() if nsplit > 1 else None, part_ml.data_ptr() if nsplit > 1 else None, nsplit,
-                    int(exact_weights)))
+                    int(exact_weights), *tail))
             if ctx.num_decode:
                 kv_len = self.fixed_kv_len or ctx.max_kv_len
                 skewed = self.fixed_skew if self.fixed_kv_len else ctx.decode_skewed
@@ -784,11 +789,12 @@ class HipOps:
                 self._need(ctx.num_decode * nsplit <= parts, "attention: more (request, run) pairs than planned for")
                 part_o = self.ws.get("attn.part_o", (parts * hq * d,), torch.float32)
                 part_ml = self.ws.get("attn.part_ml", (parts * hq * 2,), torch.float32)
-                self._ok(self.lib.psamd_attention_decode(
+                tail = (_ptr(sink), _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1]) if extras else ()
+                self._ok((self.lib.psamd_attention_decode_extras if extras else self.lib.psamd_attention_decode)(
                     s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(),
                     ctx.dec_items.data_ptr(), ctx.num_decode, ctx.item_start.data_ptr(),
                     ctx.item_end.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, nsplit, scale,
-                    win, min_run, int(exact_weights)))
+                    win, min_run, int(exact_weights), *tail))
             return
         self._ok(self.lib.psamd_attention_generic(
             s, qkv.data_ptr(), stride, out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t, ctx.positions.data_ptr(),

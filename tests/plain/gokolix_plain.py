@@ -45,13 +45,6 @@ def load_tensors(folder: Path) -> dict[str, np.ndarray]:
     return out
 
 
-def to_bf16(x: np.ndarray) -> np.ndarray:
-    """x rounded to the nearest bfloat16 (ties to even), as float64."""
-    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
-    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16 << 16
-    return u.astype(np.uint32).view(np.float32).astype(np.float64)
-
-
 # ------------------------------------------------------------------ small pieces
 
 def rms(x: np.ndarray, eps: float) -> np.ndarray:
@@ -149,7 +142,8 @@ def biased_attention(h: np.ndarray, w: dict, m: dict, eps: float) -> np.ndarray:
     k = weighted_norm(k, w["k.norm"], eps)
     rep = heads // kvh
     buckets = w["rel"].shape[0]
-    rows = np.array([[distance_bucket(i - j, buckets, m["bias_max"]) if j <= i else 0 for j in range(t)] for i in range(t)])
+    by_distance = np.array([distance_bucket(n, buckets, m["bias_max"]) for n in range(t)])
+    rows = by_distance[np.clip(np.arange(t)[:, None] - np.arange(t)[None, :], 0, None)]     # [query, key]; keys ahead are masked
     scores = np.empty((heads, t, t))
     for a in range(heads):
         scores[a] = q[:, a] @ k[:, a // rep].T * m["scale"] + w["rel"][rows, a]

@@ -1,0 +1,441 @@
+"""Gokolix on the GPU: the kernels it brought, each against a plain float32 computation in torch,
+and the model in both dtypes against the plain implementation in tests/plain/gokolix_plain.py: every
+cutting, mixed batches on reused pages and slots, contexts long enough for the attention kernels to
+cut their keys into runs, captured decode steps, generation, and the programs a user starts."""
+
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+from gokolix_configs import GOKOLIX, attention, latent, layer, model, recurrence, write_gokolix
+from plain import gokolix_plain as plain
+from prefixserve_amd.engine.batch import StepItem
+from prefixserve_amd.engine.replay import TraceReplayer
+from prefixserve_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+DEV = "cuda:0"
+F32_TOL = 3e-5
+# bfloat16: a row's largest error over its largest logit. These tiny models have peaky softmaxes and
+# sums that nearly cancel; the bars are three times what the committed configurations measure.
+BF16_MEAN, BF16_ROW = 3e-2, 1.5e-1
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from prefixserve_amd.kernels.ops import HipOps
+    from prefixserve_amd.parts.base import Workspace
+
+    return HipOps(torch.device(DEV), Workspace(torch.device(DEV)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: write_gokolix(tmp_path_factory.mktemp(f"gokolix-{name}"), name) for name in GOKOLIX}
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def rel(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def runner_for(folder, pages, dtype, slots=4, graphs=False):
+    return ModelRunner(folder, dtype=dtype, device=DEV, num_blocks=pages, max_seq_len=pages * 16, max_num_seqs=slots,
+                       use_graphs=graphs)
+
+
+class Step:
+    """The few fields of a step's context that the recurrence kernels read."""
+
+    def __init__(self, lengths, slots):
+        starts = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+        self.num_tokens, self.num_items = int(starts[-1]), len(lengths)
+        self.item_start = torch.tensor(starts, device=DEV)
+        self.slots = torch.tensor(slots, dtype=torch.int32, device=DEV)
+        self.tok_item = torch.tensor(np.repeat(np.arange(len(lengths)), lengths).astype(np.int32), device=DEV)
+
+
+# ------------------------------------------------------------------ kernels
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,heads,n,k", [(1, 3, 40, 24), (37, 2, 8, 70), (200, 5, 65, 17), (64, 1, 64, 64)])
+def test_heads_linear(ops, dtype, m, heads, n, k):
+    """Heads inside wider rows on both sides; what lies between them is left alone."""
+    x_off, x_head, o_off, o_head = 3, k + 5, 2, n + 7
+    x = rnd(m, x_off + heads * x_head, dtype=dtype, seed=1)
+    w = rnd(heads, n, k, dtype=dtype, seed=2, scale=0.3)
+    out = torch.full((m, o_off + heads * o_head + 1), 7.0, dtype=dtype, device=DEV)
+    ops.heads_linear(x, x_off, x_head, w, out, o_off, o_head)
+    want = torch.full_like(out, 7.0, dtype=torch.float32)
+    for h in range(heads):
+        want[:, o_off + h * o_head: o_off + h * o_head + n] = x[:, x_off + h * x_head: x_off + h * x_head + k].float() @ w[h].float().T
+    assert rel(out.float().cpu(), want.cpu()) < (1e-5 if dtype == torch.float32 else 1e-2)
+    assert torch.equal(out[:, :o_off].float(), want[:, :o_off]) and torch.equal(out[:, -1].float(), want[:, -1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_stream_kernels(ops, dtype):
+    x = rnd(9, 50, seed=1)
+    keep = x.clone()
+    ops.stream_affine(x, 2.5, None)
+    assert torch.equal(x, keep * 2.5)
+    row = rnd(50, seed=2)
+    ops.stream_affine(x, 1.0, row)
+    assert torch.equal(x, keep * 2.5 + row)
+    d = rnd(9, 50, dtype=dtype, seed=3)
+    ops.residual_add(x, d)
+    assert torch.equal(x, keep * 2.5 + row + d.float())
+    parts = rnd(3, 9, 50, seed=4)
+    before = x.clone()
+    ops.residual_add(x, parts)
+    assert torch.equal(x, ((before + parts[0]) + parts[1]) + parts[2])
+    both = torch.empty(9, 100, dtype=dtype, device=DEV)
+    ops.concat_to_activation(keep, row.expand(9, 50).contiguous(), both)
+    assert torch.equal(both[:, :50], keep.to(dtype)) and torch.equal(both[:, 50:], row.expand(9, 50).to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activation", ["relu", "gelu_tanh", "silu"])
+@pytest.mark.parametrize("m", [1, 8, 20, 40, 100])
+def test_gated_product_with_other_activations(ops, dtype, activation, m):
+    """Every form the gate/up product takes (fused for small steps, the library and the activation
+    kernel above) with the activation a model names."""
+    k, inter = 64, 96
+    x = rnd(m, k, dtype=dtype, seed=1)
+    w = rnd(2 * inter, k, dtype=dtype, seed=2, scale=0.2)
+    out = torch.empty(m, inter, dtype=dtype, device=DEV)
+    ops.linear_swiglu(x, w, out, activation=activation)
+    gu = x.float() @ w.float().T
+    act = {"relu": torch.relu, "silu": torch.nn.functional.silu,
+           "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh")}[activation]
+    want = act(gu[:, :inter]) * gu[:, inter:]
+    assert rel(out.float().cpu(), want.cpu()) < (2e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,hkv,d,norm_dim", [(4, 2, 48, 48), (3, 3, 16, 12), (6, 1, 160, 150)])
+def test_bias_weighted_norm_and_values_from_keys(ops, dtype, hq, hkv, d, norm_dim):
+    t, blocks = 21, 4
+    rows = rnd(t, (hq + hkv) * d, dtype=dtype, seed=1)
+    rows.view(t, hq + hkv, d)[:, :, norm_dim:] = 0            # the head's unused slots hold zeros
+    bias = rnd((hq + hkv) * d, seed=2, scale=0.5)
+    bias.view(hq + hkv, d)[:, norm_dim:] = 0
+    wq, wk = 1 + rnd(d, seed=3, scale=0.2), 1 + rnd(d, seed=4, scale=0.2)
+    kv = torch.full((blocks, 2, hkv, 16 * d), 9.0, dtype=dtype, device=DEV)
+    slots = torch.tensor(np.random.default_rng(0).permutation(blocks * 16)[:t].astype(np.int32), device=DEV)
+    pos = torch.arange(t, dtype=torch.int32, device=DEV)
+    x = rows.float().view(t, hq + hkv, d) + bias.view(hq + hkv, d)
+    normed = x * torch.rsqrt((x * x).sum(-1, keepdim=True) / norm_dim + 1e-5)
+    normed[:, :hq] *= wq
+    normed[:, hq:] *= wk
+    ops.rope_norm_kv_append(rows, hq, hkv, d, pos, None, kv, slots, norm_dim, 1e-5, bias=bias, q_weight=wq, k_weight=wk,
+                            values_from_keys=True)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert rel(rows.float().cpu(), normed.reshape(t, -1).cpu()) < tol
+    page, off = (slots // 16).long(), (slots % 16).long()
+    keys = kv[:, 0].view(blocks, hkv, 16, d)[page, :, off]
+    vals = kv[:, 1].view(blocks, hkv, d, 16)[page, :, :, off]
+    assert rel(keys.float().cpu(), normed[:, hq:].cpu()) < tol and rel(vals.float().cpu(), x[:, hq:].cpu()) < tol
+    written = torch.zeros(blocks * 16, dtype=torch.bool, device=DEV)
+    written[slots.long()] = True
+    untouched = kv[:, 0].view(blocks, hkv, 16, d).permute(0, 2, 1, 3).reshape(blocks * 16, -1)[~written]
+    assert bool((untouched == 9.0).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hq,dim,rot,rank,slots", [(3, 12, 6, 20, 32), (1, 8, 0, 16, 16), (8, 64, 16, 96, 112)])
+def test_latent_cache_write(ops, dtype, hq, dim, rot, rank, slots):
+    t, blocks = 19, 3
+    width = hq * (dim + rot) + rank + rot
+    rows = rnd(t, width + 3, dtype=dtype, seed=1)
+    q_lat = torch.full((t, hq * slots), 5.0, dtype=dtype, device=DEV)
+    w = 1 + rnd(rank, seed=2, scale=0.2)
+    table = torch.stack([torch.cos(rnd(40, max(rot // 2, 1), seed=3)), torch.sin(rnd(40, max(rot // 2, 1), seed=3))], dim=-1).contiguous()
+    pos = torch.tensor(np.random.default_rng(1).integers(0, 40, t).astype(np.int32), device=DEV)
+    kv = torch.full((blocks, 2, 1, 16 * slots), 9.0, dtype=dtype, device=DEV)
+    ws = torch.tensor(np.random.default_rng(2).permutation(blocks * 16)[:t].astype(np.int32), device=DEV)
+    ops.latent_kv_append(rows, q_lat, hq, dim, rot, rank, slots, pos, table if rot else None, w, 1e-5, kv, ws)
+
+    def turn(v):
+        cs = table[pos.long()]
+        while cs.dim() - 1 < v.dim():
+            cs = cs.unsqueeze(1)
+        a, b = v[..., 0::2], v[..., 1::2]
+        out = torch.empty_like(v)
+        out[..., 0::2] = a * cs[..., 0] - b * cs[..., 1]
+        out[..., 1::2] = b * cs[..., 0] + a * cs[..., 1]
+        return out
+
+    low = rows[:, hq * (dim + rot): width].float()
+    c = low[:, :rank] * torch.rsqrt((low[:, :rank] ** 2).mean(-1, keepdim=True) + 1e-5) * w
+    key = torch.zeros(t, slots, device=DEV)
+    key[:, :rank] = c
+    val = key.clone()
+    q = rows[:, : hq * (dim + rot)].float().view(t, hq, dim + rot)
+    want_q = torch.full((t, hq, slots), 5.0, device=DEV)
+    want_q[:, :, rank:] = 0
+    if rot:
+        key[:, rank: rank + rot] = turn(low[:, rank:])
+        want_q[:, :, rank: rank + rot] = turn(q[:, :, dim:])
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    page, off = (ws // 16).long(), (ws % 16).long()
+    assert rel(kv[:, 0].view(blocks, 16, slots)[page, off].float().cpu(), key.cpu()) < tol
+    assert rel(kv[:, 1].view(blocks, slots, 16)[page, :, off].float().cpu(), val.cpu()) < tol
+    assert rel(q_lat.float().view(t, hq, slots).cpu(), want_q.cpu()) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,blocks,taps", [(48, 3, 3), (40, 1, 1), (300, 4, 5)])
+def test_convolution_and_recurrence_continue_from_their_slot(ops, dtype, width, blocks, taps):
+    """Three requests in slots full of junk except where they start; a second step continues two of
+    them (one with a single token, one with fewer tokens than taps) beside a new one."""
+    bw = width // blocks
+    conv_w, conv_b = rnd(width, taps, seed=1, scale=0.5), rnd(width, seed=2, scale=0.3)
+    xb, yb = rnd(width, seed=3, scale=0.3), rnd(width, seed=4, scale=0.3)
+    wg, gb = rnd(blocks, 2 * bw, bw, seed=5, scale=0.4), rnd(blocks * 2 * bw, seed=6, scale=0.5)
+    decay = -8.0 * torch.nn.functional.softplus(rnd(width, seed=7))
+    state = torch.full((5, taps * width), 1e30, device=DEV)
+    seqs = {s: rnd(n, 2 * width, dtype=dtype, seed=10 + s) for s, n in ((4, 9), (1, 14), (2, 6), (0, 5))}
+
+    def plain_run(rows):                                   # one request, whole
+        n = rows.shape[0]
+        y = torch.nn.functional.gelu(rows[:, :width].float() + yb, approximate="tanh")
+        x = torch.cat([torch.zeros(taps - 1, width, device=DEV), rows[:, width:].float() + xb])
+        u = conv_b + sum(conv_w[:, j] * x[j: j + n] for j in range(taps))
+        g = torch.einsum("tbi,boi->tbo", u.view(n, blocks, bw), wg) + gb.view(blocks, 2 * bw)
+        r, i = torch.sigmoid(g[:, :, :bw]).reshape(n, width), torch.sigmoid(g[:, :, bw:]).reshape(n, width)
+        a = torch.exp(decay * r)
+        s, out = torch.zeros(width, device=DEV), []
+        for k in range(n):
+            s = a[k] * s + torch.sqrt(1 - a[k] ** 2) * i[k] * u[k]
+            out.append(s * y[k])
+        return torch.stack(out)
+
+    def step(pieces):                                      # [(slot, rows)] as one batch
+        ctx = Step([p.shape[0] for _, p in pieces], [s for s, _ in pieces])
+        rows = torch.cat([p for _, p in pieces]).contiguous()
+        u = torch.empty(ctx.num_tokens, width, device=DEV)
+        ops.causal_conv(rows, width, xb, conv_w, conv_b, u, state, ctx)
+        gates = torch.empty(ctx.num_tokens, 2 * width, device=DEV)
+        ops.heads_linear(u, 0, bw, wg, gates, 0, 2 * bw)
+        out = torch.empty(ctx.num_tokens, width, dtype=dtype, device=DEV)
+        ops.gated_scan(gates, gb, u, decay, rows, 0, width, yb, xb, out, state, ctx, blocks, taps)
+        return out.float()
+
+    for s in (4, 1, 2):
+        state[s].zero_()                                   # what the runner does for a request at position 0
+    first = step([(4, seqs[4][:7]), (1, seqs[1][:3]), (2, seqs[2])])
+    state[0].zero_()
+    second = step([(1, seqs[1][3:4]), (0, seqs[0]), (4, seqs[4][7:])])
+    third = step([(1, seqs[1][4:])])
+    got = {4: torch.cat([first[:7], second[6:]]), 1: torch.cat([first[7:10], second[:1], third]), 2: first[10:], 0: second[1:6]}
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for s, rows in seqs.items():
+        assert rel(got[s].cpu(), plain_run(rows).cpu()) < tol, s
+    assert bool((state[3] == 1e30).all())                  # a slot nobody used
+
+
+# ------------------------------------------------------------------ whole models
+
+LENGTHS = [70, 33, 97, 18, 64, 45, 1, 52, 2, 81, 29, 3]
+
+
+def check_rows(errors, dtype):
+    if dtype == "float32":
+        assert max(errors) < F32_TOL
+    else:
+        assert float(np.mean(errors)) < BF16_MEAN and max(errors) < BF16_ROW, (float(np.mean(errors)), max(errors))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(GOKOLIX))
+def test_every_cutting_matches_the_plain_model(name, dtype, folders):
+    rng = np.random.default_rng(4)
+    reqs = [rng.integers(0, GOKOLIX[name]["vocab"], n).tolist() for n in LENGTHS]
+    pm = plain.PlainGokolix(folders[name])
+    truth = [pm.logits(t) for t in reqs]
+    runner = runner_for(folders[name], 32, dtype)
+    for build in (traces.whole, traces.decode_tail, traces.portions):
+        steps, expect = build(reqs)
+        errors: list = []
+        traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, 1.0, errors)
+        check_rows(errors, dtype)
+    steps, expect, peak = traces.mixed(reqs, max_live=3, seed=2)
+    small = runner_for(folders[name], peak // 16, dtype, slots=3)
+    for t in small.pools.tensors:
+        t.fill_(3e4)                                        # a page that is used again never holds zeros
+    for s in small.states.values():
+        s.fill_(1e30)
+    rp = TraceReplayer(small)
+    errors = []
+    traces.compare(rp.run_step, steps, expect, truth, 1.0, errors)
+    check_rows(errors, dtype)
+    assert all(rp.cache.num_free(g) == peak // 16 for g in range(rp.cache.num_groups))
+
+
+def test_cuttings_agree_with_each_other_in_32_bit(folders):
+    """A position's 32-bit logits do not depend on how its prompt was cut, beyond rounding."""
+    toks = np.random.default_rng(8).integers(0, 96, 90).tolist()
+    runner = runner_for(folders["A"], 16, "float32")
+    rows = {}
+    for build in (traces.whole, traces.decode_tail, traces.portions):
+        steps, expect = build([toks])
+        rp = TraceReplayer(runner)
+        got = np.concatenate([r for r in (rp.run_step(s) for s in steps) if r is not None])
+        rows[build.__name__] = {p: got[k] for k, (_, p) in enumerate(e for exp in expect for e in exp)}
+    for p in rows["decode_tail"]:
+        assert rel(rows["decode_tail"][p], rows["whole"][p]) < 5e-6 and rel(rows["portions"][p], rows["whole"][p]) < 5e-6
+
+
+def peaky(tensors):
+    for name, t in tensors.items():
+        if name.endswith(".sink"):
+            t.copy_(torch.full_like(t, 2.0))
+        if name.endswith(".rel"):
+            t.mul_(4.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_contexts_without_windows(dtype, tmp_path):
+    """No window: 2,100 keys, so that the decode attention and the attention of a short portion cut
+    their keys into runs and the sink joins in the merge; score scales under which single keys
+    hundreds of tokens back carry the weight. Attention alone, then latent attention alone."""
+    for k, mixer in enumerate((attention(4, 2, 32, 1.5, 300, 24), latent(4, 16, 8, 16, 24, 1.5, 10000.0))):
+        folder = write_gokolix(tmp_path / f"m{k}", model(80, 64, 1e-5, 2.0, [layer(mixer, 32)]), seed=3 + k, edit=peaky)
+        toks = np.random.default_rng(5).integers(0, 80, 2110).tolist()
+        truth = plain.PlainGokolix(folder).logits(toks)
+        runner = runner_for(folder, 140, dtype)
+        steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:2080], "want": [100, 2079]}], "end": []},
+                 {"step": 1, "entries": [{"id": "a", "tokens": toks[2080:2100], "want": list(range(20))}], "end": []}]
+        steps += [{"step": 2 + i, "entries": [{"id": "a", "tokens": [toks[2100 + i]], "want": [0]}], "end": []} for i in range(10)]
+        expect = [[(0, 100), (0, 2079)], [(0, p) for p in range(2080, 2100)]] + [[(0, 2100 + i)] for i in range(10)]
+        errors: list = []
+        traces.compare(TraceReplayer(runner).run_step, steps, expect, [truth], 1.0, errors)
+        check_rows(errors, dtype)
+        far = np.abs(plain.PlainGokolix(folder).logits(toks[1500:])[-1] - truth[-1]).max() / np.abs(truth[-1]).max()
+        assert far > 100 * F32_TOL                          # the keys far back matter to the last row
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_through_graphs_without_a_recurrence(dtype, tmp_path):
+    """A model of attention layers alone keeps no state, so its decode steps are captured: the
+    replays give what single launches give."""
+    cfg = model(90, 64, 1e-5, 2.0, [layer(attention(4, 2, 16, 0.5, 20, 12, window=24), 48),
+                                    layer(latent(2, 16, 8, 16, 24, 0.4, 1000.0, window=40), 48)], loop=(0, 2, 2))
+    folder = write_gokolix(tmp_path, cfg, seed=4)
+    toks = np.random.default_rng(2).integers(0, 90, 120).tolist()
+    truth = plain.PlainGokolix(folder).logits(toks)
+    runner = runner_for(folder, 16, dtype, graphs=True)
+    assert runner.use_graphs and not runner.states
+    steps, expect = traces.decode_tail([toks], tail=70)
+    errors: list = []
+    traces.compare(TraceReplayer(runner).run_step, steps, expect, [truth], 1.0, errors)
+    check_rows(errors, dtype)
+    assert runner._graphs
+
+
+def test_greedy_generation_through_the_entry_point(folders):
+    from prefixserve_amd.engine.engine import Engine, EngineConfig
+    from prefixserve_amd.generation import generate
+
+    pm = plain.PlainGokolix(folders["A"])
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(0, 96, n).tolist() for n in (5, 23, 40, 9, 31)]
+    eng = Engine(EngineConfig(model_path=str(folders["A"]), dtype="float32", max_num_seqs=3, max_prefill_tokens=16,
+                              max_seq_len=128, num_blocks=14))
+    outs, _ = generate(eng, prompts, 12, temperature=0.0, ignore_eos=True)
+    for p, o in zip(prompts, outs):
+        assert list(o.tokens) == pm.greedy(p, 12)
+
+
+def test_trace_run_and_the_command_line_as_programs(folders, tmp_path):
+    rng = np.random.default_rng(7)
+    reqs = [rng.integers(0, 130, n).tolist() for n in (40, 70, 25, 90, 33)]
+    pm = plain.PlainGokolix(folders["B"])
+    truth = [pm.logits(t) for t in reqs]
+    steps, expect, peak = traces.mixed(reqs, max_live=3, seed=5)
+    env = {k: v for k, v in os.environ.items()}
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / f"out-{dtype}"
+        proc = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(folders["B"]), "--dtype", dtype, "--out", str(out),
+                               "--max-tokens", str(peak)], input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+                              capture_output=True, env=env, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        errors = []
+        for s, exp in zip(steps, expect):
+            if exp:
+                got = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(exp), -1)
+                errors += [rel(row, truth[i][p]) for row, (i, p) in zip(got, exp)]
+        check_rows(errors, dtype)
+    prompt = [5, 17, 3, 90, 41, 7, 7, 19, 0, 64, 11]
+    proc = subprocess.run(
+        [sys.executable, "-m", "prefixserve_amd.cli", "generate", "--model", str(folders["B"]), "--dtype", "float32",
+         "--max-seq-len", "128", "--num-blocks", "16", "--max-running-requests", "2", "--chunked-prefill-size", "5",
+         "--max-tokens", "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt))],
+        capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert json.loads(proc.stdout.strip().splitlines()[-1])["outputs"][0]["tokens"] == pm.greedy(prompt, 6)
+
+
+def random_gokolix(rng) -> dict:
+    """A configuration drawn at random: widths that are no multiples of 8 or 16, one to three layers
+    of every kind in any order, with and without feed-forward, windows and scaling, any stretch repeated."""
+    width = int(rng.choice([40, 72, 100, 136]))
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        kind = int(rng.integers(0, 3))
+        window = None if rng.random() < 0.3 else int(rng.choice([1, 2, 7, 16, 33, 70]))
+        if kind == 0:
+            kvh = int(rng.choice([1, 2, 3]))
+            buckets = int(rng.choice([2, 5, 8, 32]))
+            mixer = attention(kvh * int(rng.choice([1, 2, 4])), kvh, int(rng.choice([8, 20, 32, 48, 72])), float(rng.choice([0.1, 0.5, 1.0])),
+                              float(buckets // 2 + rng.choice([1, 3.5, 40])), buckets, window)
+        elif kind == 1:
+            rot = int(rng.choice([0, 2, 8, 16]))
+            scaling = None if rng.random() < 0.4 else {"factor": float(rng.choice([2.0, 8.0, 40.0])), "original": int(rng.choice([16, 64, 512])),
+                                                        "fast": float(rng.choice([4.0, 32.0])), "slow": float(rng.choice([0.25, 1.0, 2.0]))}
+            mixer = latent(int(rng.choice([1, 3, 8])), int(rng.choice([4, 16, 40])), rot, int(rng.choice([6, 16, 24])),
+                           int(rng.choice([8, 30, 64, 100])), float(rng.choice([0.1, 0.4])), float(rng.choice([10.0, 10000.0])), scaling, window)
+        else:
+            blocks = int(rng.choice([1, 2, 5]))
+            mixer = recurrence(blocks * int(rng.choice([4, 9, 16])), blocks, int(rng.choice([1, 2, 4, 7])))
+        layers.append(layer(mixer, None if rng.random() < 0.25 else int(rng.choice([12, 40, 64]))))
+    loop = None
+    if rng.random() < 0.7:
+        a = int(rng.integers(0, len(layers)))
+        loop = (a, int(rng.integers(a + 1, len(layers) + 1)), int(rng.integers(1, 4)))
+    return model(int(rng.choice([50, 131, 256])), width, float(rng.choice([1e-5, 1e-6])), float(rng.choice([1.0, 4.0, 12.5])), layers, loop)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_configurations_in_both_dtypes(seed, tmp_path):
+    rng = np.random.default_rng(100 + seed)
+    cfg = random_gokolix(rng)
+    folder = write_gokolix(tmp_path, cfg, seed=seed)
+    reqs = [rng.integers(0, cfg["vocab"], n).tolist() for n in (90, 17, 45, 3)]
+    pm = plain.PlainGokolix(folder)
+    truth = [pm.logits(t) for t in reqs]
+    steps, expect, peak = traces.mixed(reqs, max_live=3, seed=seed)
+    for dtype in ("float32", "bfloat16"):
+        errors: list = []
+        traces.compare(TraceReplayer(runner_for(folder, peak // 16, dtype, slots=3)).run_step, steps, expect, truth, 1.0, errors)
+        if dtype == "float32":
+            assert max(errors) < F32_TOL, (cfg, max(errors))
+        else:
+            assert float(np.mean(errors)) < 2 * BF16_MEAN, (cfg, float(np.mean(errors)))
