@@ -91,9 +91,42 @@ def radivik_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
     return radivik, llama
 
 
+# Gokolix at sizes that resemble real layers, beside the Llama decoder of equal size: same width, the
+# attention layers' head counts and head size, the same inner feed-forward size and as many layer runs
+# (a repeated stretch counts every pass). Four layers: attention, recurrence, latent attention, attention;
+# the first two are passed through twice. The latent cache entry (rank + rotated part) is 256 wide, the
+# largest head the attention kernels take.
+GOKOLIX_SIZES = {
+    "gokolix-w2048-h32x64-ff8192": dict(width=2048, heads=32, kv_heads=8, dim=64, ff=8192, window=1024, rec_width=2048, rec_blocks=16,
+                                        lat_heads=16, lat_dim=128, lat_rot=64, lat_vdim=128, rank=192),
+    "gokolix-w4096-h32x128-ff14336": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, window=4096, rec_width=4096,
+                                          rec_blocks=32, lat_heads=32, lat_dim=128, lat_rot=64, lat_vdim=128, rank=192),
+}
+
+
+def gokolix_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
+    """(Gokolix config.json, the Llama config.json of equal size). ``layers`` is not used: the
+    pattern of four layers with its first two passed through twice is six layer runs."""
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    att = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"], "scale": size["dim"] ** -0.5,
+        "bias_max": 512, "buckets": 32, "mask": {"size": size["window"]}}}
+    rec = {"type": "rglru", "mlp": mlp, "mixer": {"width": size["rec_width"], "blocks": size["rec_blocks"], "conv": 4}}
+    lat = {"type": "latent_attention", "mlp": mlp, "mixer": {
+        "heads": size["lat_heads"], "dim": size["lat_dim"], "rot_dim": size["lat_rot"], "vdim": size["lat_vdim"], "kv_rank": size["rank"],
+        "scale": (size["lat_dim"] + size["lat_rot"]) ** -0.5, "mask": {"size": size["window"]},
+        "rot": {"base": 10000.0, "dims": size["lat_rot"], "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    gokolix = {"architecture": "Gokolix", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": 8.0},
+               "layers": [att, rec, lat, att], "loop": {"start": 0, "stop": 2, "times": 2}}
+    llama = dict(LLAMA_1B, vocab_size=vocab, hidden_size=size["width"], intermediate_size=size["ff"], num_hidden_layers=6,
+                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                 tie_word_embeddings=True)
+    return gokolix, llama
+
+
 def compare_designs(args) -> int:
-    """Prefill and decode throughput of Radivik layers beside Llama layers of equal size, through
-    the same runner and step function. One JSON line; the default benchmark is not run."""
+    """Prefill and decode throughput of another design's layers (Radivik, Gokolix) beside Llama layers of
+    equal size, through the same runner and step function. One JSON line; the default benchmark is not run."""
     import numpy as np
     import torch
 
@@ -104,14 +137,20 @@ def compare_designs(args) -> int:
     rng = np.random.default_rng(0)
     vocab, layers = 32000, args.layers or 4
     prompt, batch, context = args.prompt_len, args.batch, args.context
-    sizes = RADIVIK_SIZES if args.compare == "all" else {args.compare: RADIVIK_SIZES[args.compare]}
+    if args.compare in GOKOLIX_SIZES or args.compare == "gokolix":
+        design, pair_of = "gokolix", gokolix_pair
+        sizes = GOKOLIX_SIZES if args.compare == "gokolix" else {args.compare: GOKOLIX_SIZES[args.compare]}
+    else:
+        design, pair_of = "radivik", radivik_pair
+        sizes = RADIVIK_SIZES if args.compare == "all" else {args.compare: RADIVIK_SIZES[args.compare]}
     results = {}
 
     def measure(folder) -> dict:
         pages_per = -(-context // 16)
         runner = ModelRunner(folder, dtype=args.dtype, num_blocks=(batch + 1) * pages_per + 8, max_seq_len=context,
-                             max_num_seqs=max(batch, 2), max_prefill_tokens=prompt, use_graphs=not args.no_graphs)
+                             max_num_seqs=max(batch + 1, 2), max_prefill_tokens=prompt, use_graphs=not args.no_graphs)
         groups = len(runner.num_blocks_per_group)
+        # Every request has its own pages and its own state slot (the prompt's request takes the last).
         tables = [[list(range(b * pages_per, (b + 1) * pages_per)) for _ in range(groups)] for b in range(batch + 1)]
         toks = rng.integers(0, vocab, prompt)
 
@@ -124,7 +163,7 @@ def compare_designs(args) -> int:
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) / reps
 
-        whole = lambda: runner.step([StepItem("p", toks, 0, tables[batch], 0, (prompt - 1,))])
+        whole = lambda: runner.step([StepItem("p", toks, 0, tables[batch], batch, (prompt - 1,))])
         t_prefill = timed(whole, args.prefill_reps)
         fill = context - args.steps - args.warmup - 2
         for b in range(batch):                                  # every request's cache, filled in portions
@@ -160,17 +199,17 @@ def compare_designs(args) -> int:
 
     with tempfile.TemporaryDirectory(prefix="psamd_compare_") as tmp:
         for name, size in sizes.items():
-            radivik, llama = radivik_pair(size, layers, vocab)
+            other, llama = pair_of(size, layers, vocab)
             results[name] = {}
-            for design, cfg in (("radivik", radivik), ("llama", llama)):
-                if args.compare_only not in ("both", design):
+            for which, cfg in ((design, other), ("llama", llama)):
+                if args.compare_only not in ("both", which):
                     continue
-                folder = write_random_model(Path(tmp) / f"{name}-{design}", cfg, seed=0)
-                results[name][design] = measure(folder)
+                folder = write_random_model(Path(tmp) / f"{name}-{which}", cfg, seed=0)
+                results[name][which] = measure(folder)
             both = results[name]
             if len(both) == 2:
-                both["radivik_over_llama"] = {k: both["radivik"][k] / both["llama"][k] for k in ("prefill_tok_s", "decode_tok_s")}
-    print(json.dumps({"metric": "radivik_beside_llama_of_equal_size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
+                both[f"{design}_over_llama"] = {k: both[design][k] / both["llama"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+    print(json.dumps({"metric": f"{design}_beside_llama_of_equal_size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
                       "data": "synthetic: seeded uniform-random token ids, seeded random weights",
                       "config": {"layers": layers, "vocab": vocab, "prompt_len": prompt, "decode_batch": batch,
                                  "context": context, "steps": args.steps, "warmup": args.warmup},
@@ -214,10 +253,11 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
-    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"], default=None,
-                    help="instead of the benchmark: Radivik layers of this size beside Llama layers of equal size "
-                         "(prefill of --prompt-len tokens, decoding at --batch in --context; --layers, default 4)")
-    ap.add_argument("--compare-only", choices=["both", "radivik", "llama"], default="both")
+    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"] + sorted(GOKOLIX_SIZES) + ["gokolix"], default=None,
+                    help="instead of the benchmark: Radivik or Gokolix layers of this size ('all': every Radivik size, "
+                         "'gokolix': every Gokolix size) beside Llama layers of equal size (prefill of --prompt-len tokens, "
+                         "decoding at --batch in --context; --layers, default 4, for Radivik)")
+    ap.add_argument("--compare-only", choices=["both", "radivik", "gokolix", "llama"], default="both")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

@@ -96,11 +96,15 @@ int psamd_causal_conv(void* stream, const void* in, int act_dtype, int64_t in_ro
 // gate_b), i = sigmoid(gates[t, b, bw + c'] + gate_b) (gates [tokens, blocks, 2 * bw], c = b * bw + c'),
 // log a = decay[c] * r: S = a S + sqrt(1 - a^2) i u[t, c]; out[t, c] = S * gelu_tanh(y[t, c] + y_bias[c]).
 // S lives in state[slot, (taps - 1) * width + c]; behind the scan the state's saved inputs become the
-// item's last taps - 1 values of x[t, c] + x_bias[c].
+// item's last taps - 1 values of x[t, c] + x_bias[c]. tiles == NULL: every item token after token.
+// Otherwise the step packer's lists: tiles[k] = (item, first token) of the n_tiles tiles of `tile` tokens
+// that the items of more than one token are cut into (summed up tile by tile, then run side by side;
+// carry: 3 * n_tiles * width floats), and singles: the n_singles items of one token.
 int psamd_gated_scan(void* stream, const float* gates, const float* gate_b, const float* u, const float* decay,
                      const void* y, const void* x, int act_dtype, int64_t in_row, const float* y_bias,
                      const float* x_bias, void* out, float* state, int64_t state_row, const int32_t* item_start,
-                     const int32_t* slots, int items, int width, int blocks, int taps);
+                     const int32_t* slots, int items, const int32_t* tiles, int n_tiles, int tile,
+                     const int32_t* singles, int n_singles, float* carry, int width, int blocks, int taps);
 
 // Mixture of experts. Router: z = x w_router^T in float (x in x_dtype, w_router float [E, K]), score =
 // sigmoid(z); chosen[t, :] = the top largest scores' experts (lower index among equals, largest

@@ -43,37 +43,19 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
 
+// One token of the recurrence: the decay a and what flows in, from the gates' sums.
+__device__ __forceinline__ void scan_terms(float gr, float gi, float dec, float u, float& a, float& inflow) {
+  const float r = sigmoid_f(gr), g = sigmoid_f(gi);
+  const float la = dec * r;
+  a = expf(la);
+  inflow = sqrtf(-expm1f(2.f * la)) * g * u;
+}
+
+// The state's saved inputs after an item's step: the last taps - 1 of (saved before, then this step's).
 template <typename A>
-__global__ __launch_bounds__(256) void gated_scan_kernel(
-    const float* __restrict__ gates, const float* __restrict__ gate_b, const float* __restrict__ u,
-    const float* __restrict__ decay, const A* __restrict__ y, const A* __restrict__ x, int64_t in_row,
-    const float* __restrict__ y_bias, const float* __restrict__ x_bias, A* __restrict__ out, float* __restrict__ state,
-    int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots, int width, int blocks,
-    int taps) {
-  const int item = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
-  if (c >= width) return;
-  const int bw = width / blocks;
-  const int b = c / bw, cb = c - b * bw;
-  const int64_t s0 = item_start[item], s1 = item_start[item + 1];
-  float* st = state + static_cast<int64_t>(slots[item]) * state_row;
-  const int64_t g_off = static_cast<int64_t>(b) * 2 * bw + cb;
-  const float br = gate_b[g_off], bi = gate_b[g_off + bw];
-  const float dec = decay[c], yb = y_bias[c];
-  float S = st[static_cast<int64_t>(taps - 1) * width + c];
-  for (int64_t t = s0; t < s1; ++t) {
-    const float r = sigmoid_f(gates[t * 2 * width + g_off] + br);
-    const float g = sigmoid_f(gates[t * 2 * width + g_off + bw] + bi);
-    const float la = dec * r;
-    const float a = expf(la);
-    const float step = sqrtf(-expm1f(2.f * la));
-    S = fmaf(a, S, step * g * u[t * width + c]);
-    out[t * width + c] = from_float<A>(S * gelu_tanh_f(to_float<A>(y[t * in_row + c]) + yb));
-  }
-  st[static_cast<int64_t>(taps - 1) * width + c] = S;
-  // The inputs the next step's convolution reaches back to: the last taps - 1 of (saved, then this step's).
-  const int n = static_cast<int>(s1 - s0), keep = taps - 1;
-  const float xb = x_bias[c];
+__device__ __forceinline__ void save_inputs(float* st, const A* x, int64_t in_row, int64_t s0, int n, int taps, int width,
+                                            int c, float xb) {
+  const int keep = taps - 1;
   float next[kMaxTaps];
 #pragma unroll
   for (int k = 0; k < kMaxTaps; ++k) {
@@ -85,6 +67,95 @@ __global__ __launch_bounds__(256) void gated_scan_kernel(
 #pragma unroll
   for (int k = 0; k < kMaxTaps; ++k)
     if (k < keep) st[static_cast<int64_t>(k) * width + c] = next[k];
+}
+
+// The whole of each listed item, token after token: a thread per (item, channel). For items of one
+// token (decoding), where there is nothing to share out. `list` (or NULL: every item) names the items.
+template <typename A>
+__global__ __launch_bounds__(256) void gated_scan_kernel(
+    const float* __restrict__ gates, const float* __restrict__ gate_b, const float* __restrict__ u,
+    const float* __restrict__ decay, const A* __restrict__ y, const A* __restrict__ x, int64_t in_row,
+    const float* __restrict__ y_bias, const float* __restrict__ x_bias, A* __restrict__ out, float* __restrict__ state,
+    int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ list, int width, int blocks, int taps) {
+  const int item = list != nullptr ? list[blockIdx.x] : blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int bw = width / blocks;
+  const int b = c / bw, cb = c - b * bw;
+  const int64_t s0 = item_start[item], s1 = item_start[item + 1];
+  float* st = state + static_cast<int64_t>(slots[item]) * state_row;
+  const int64_t g_off = static_cast<int64_t>(b) * 2 * bw + cb;
+  const float br = gate_b[g_off], bi = gate_b[g_off + bw];
+  const float dec = decay[c], yb = y_bias[c];
+  float S = st[static_cast<int64_t>(taps - 1) * width + c];
+  for (int64_t t = s0; t < s1; ++t) {
+    float a, inflow;
+    scan_terms(gates[t * 2 * width + g_off] + br, gates[t * 2 * width + g_off + bw] + bi, dec, u[t * width + c], a, inflow);
+    S = fmaf(a, S, inflow);
+    out[t * width + c] = from_float<A>(S * gelu_tanh_f(to_float<A>(y[t * in_row + c]) + yb));
+  }
+  st[static_cast<int64_t>(taps - 1) * width + c] = S;
+  save_inputs<A>(st, x, in_row, s0, static_cast<int>(s1 - s0), taps, width, c, x_bias[c]);
+}
+
+// Items of more than one token, cut into the step's tiles of `tile` tokens (tiles[k] = (item, first
+// token of the tile within the item); the tiles of an item follow each other): a thread per (tile,
+// channel). The recurrence S <- a S + b is linear in S, so a tile can be summed up from S = 0 as the
+// pair (product of its a, its own sum): pass 0 leaves that pair per tile and channel, and the state the
+// item started from; pass 1 folds the pairs of the tiles in front of its own (in order, from the
+// item's starting state), runs its tile from there and writes the outputs; the item's last tile
+// leaves the new state in the slot.
+template <typename A, int PASS>
+__global__ __launch_bounds__(256) void gated_scan_tiles_kernel(
+    const float* __restrict__ gates, const float* __restrict__ gate_b, const float* __restrict__ u,
+    const float* __restrict__ decay, const A* __restrict__ y, const A* __restrict__ x, int64_t in_row,
+    const float* __restrict__ y_bias, const float* __restrict__ x_bias, A* __restrict__ out, float* __restrict__ state,
+    int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ tiles, int tile, float* __restrict__ carry, int n_tiles, int width, int blocks, int taps) {
+  const int k = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int item = tiles[2 * k], q0 = tiles[2 * k + 1];
+  const int bw = width / blocks;
+  const int b = c / bw, cb = c - b * bw;
+  const int64_t s0 = item_start[item];
+  const int len = static_cast<int>(item_start[item + 1] - s0);
+  const int n = min(tile, len - q0);
+  const int64_t g_off = static_cast<int64_t>(b) * 2 * bw + cb;
+  const float br = gate_b[g_off], bi = gate_b[g_off + bw];
+  const float dec = decay[c];
+  float* st = state + static_cast<int64_t>(slots[item]) * state_row;
+  float* prod = carry;                                          // [n_tiles][width]
+  float* sum = carry + static_cast<int64_t>(n_tiles) * width;   // [n_tiles][width]
+  float* begin = carry + 2LL * n_tiles * width;                 // [n_tiles][width]: the item's starting state, at its first tile
+  if (PASS == 0) {
+    float P = 1.f, B = 0.f;
+    for (int64_t t = s0 + q0; t < s0 + q0 + n; ++t) {
+      float a, inflow;
+      scan_terms(gates[t * 2 * width + g_off] + br, gates[t * 2 * width + g_off + bw] + bi, dec, u[t * width + c], a, inflow);
+      B = fmaf(a, B, inflow);
+      P *= a;
+    }
+    prod[static_cast<int64_t>(k) * width + c] = P;
+    sum[static_cast<int64_t>(k) * width + c] = B;
+    if (q0 == 0) begin[static_cast<int64_t>(k) * width + c] = st[static_cast<int64_t>(taps - 1) * width + c];
+    return;
+  }
+  const int first = k - q0 / tile;
+  float S = begin[static_cast<int64_t>(first) * width + c];
+  for (int j = first; j < k; ++j) S = fmaf(prod[static_cast<int64_t>(j) * width + c], S, sum[static_cast<int64_t>(j) * width + c]);
+  const float yb = y_bias[c];
+  for (int64_t t = s0 + q0; t < s0 + q0 + n; ++t) {
+    float a, inflow;
+    scan_terms(gates[t * 2 * width + g_off] + br, gates[t * 2 * width + g_off + bw] + bi, dec, u[t * width + c], a, inflow);
+    S = fmaf(a, S, inflow);
+    out[t * width + c] = from_float<A>(S * gelu_tanh_f(to_float<A>(y[t * in_row + c]) + yb));
+  }
+  if (q0 + n == len) {
+    st[static_cast<int64_t>(taps - 1) * width + c] = S;
+    save_inputs<A>(st, x, in_row, s0, len, taps, width, c, x_bias[c]);
+  }
 }
 
 }  // namespace psamd
@@ -113,30 +184,54 @@ extern "C" int psamd_causal_conv(void* stream, const void* in, int act_dtype, in
   return check_launch("psamd_causal_conv");
 }
 
+template <typename A>
+static int launch_scan(hipStream_t s, const float* gates, const float* gate_b, const float* u, const float* decay,
+                       const void* y, const void* x, int64_t in_row, const float* y_bias, const float* x_bias, void* out,
+                       float* state, int64_t state_row, const int32_t* item_start, const int32_t* slots, int items,
+                       const int32_t* tiles, int n_tiles, int tile, const int32_t* singles, int n_singles, float* carry,
+                       int width, int blocks, int taps) {
+  const unsigned cb = static_cast<unsigned>(ceil_div(width, 256));
+  const A* yp = static_cast<const A*>(y);
+  const A* xp = static_cast<const A*>(x);
+  A* op = static_cast<A*>(out);
+  if (tiles == nullptr) {       // every item whole, token after token
+    gated_scan_kernel<A><<<dim3(items, cb), dim3(256), 0, s>>>(gates, gate_b, u, decay, yp, xp, in_row, y_bias, x_bias, op, state,
+                                                            state_row, item_start, slots, nullptr, width, blocks, taps);
+    return check_launch("psamd_gated_scan");
+  }
+  if (n_tiles > 0) {
+    gated_scan_tiles_kernel<A, 0><<<dim3(n_tiles, cb), dim3(256), 0, s>>>(gates, gate_b, u, decay, yp, xp, in_row, y_bias, x_bias,
+                                                                      op, state, state_row, item_start, slots, tiles, tile,
+                                                                      carry, n_tiles, width, blocks, taps);
+    gated_scan_tiles_kernel<A, 1><<<dim3(n_tiles, cb), dim3(256), 0, s>>>(gates, gate_b, u, decay, yp, xp, in_row, y_bias, x_bias,
+                                                                      op, state, state_row, item_start, slots, tiles, tile,
+                                                                      carry, n_tiles, width, blocks, taps);
+  }
+  if (n_singles > 0)
+    gated_scan_kernel<A><<<dim3(n_singles, cb), dim3(256), 0, s>>>(gates, gate_b, u, decay, yp, xp, in_row, y_bias, x_bias, op,
+                                                                state, state_row, item_start, slots, singles, width, blocks, taps);
+  return check_launch("psamd_gated_scan");
+}
+
 extern "C" int psamd_gated_scan(void* stream, const float* gates, const float* gate_b, const float* u, const float* decay,
                                 const void* y, const void* x, int act_dtype, int64_t in_row, const float* y_bias,
                                 const float* x_bias, void* out, float* state, int64_t state_row,
-                                const int32_t* item_start, const int32_t* slots, int items, int width, int blocks,
-                                int taps) {
+                                const int32_t* item_start, const int32_t* slots, int items, const int32_t* tiles,
+                                int n_tiles, int tile, const int32_t* singles, int n_singles, float* carry, int width,
+                                int blocks, int taps) {
   PSAMD_REQUIRE(items >= 0 && width > 0 && blocks > 0 && width % blocks == 0, "bad sizes");
   PSAMD_REQUIRE(taps >= 1 && taps <= kMaxTaps, "at most 16 taps");
   PSAMD_REQUIRE(in_row >= width && state_row >= static_cast<int64_t>(taps) * width, "rows too short");
   PSAMD_REQUIRE(ceil_div(width, 256) <= 65535, "too large for one launch");
+  PSAMD_REQUIRE(tiles == nullptr || (n_tiles >= 0 && n_singles >= 0 && tile >= 1 && (n_tiles == 0 || carry != nullptr) &&
+                                     (n_singles == 0 || singles != nullptr)), "tiles need their size, the singles' list and room for the carries");
   if (items == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(items), static_cast<unsigned>(ceil_div(width, 256)));
-  if (act_dtype == kBF16) {
-    gated_scan_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(gates, gate_b, u, decay, static_cast<const bf16_t*>(y),
-                                                        static_cast<const bf16_t*>(x), in_row, y_bias, x_bias,
-                                                        static_cast<bf16_t*>(out), state, state_row, item_start, slots,
-                                                        width, blocks, taps);
-  } else if (act_dtype == kF32) {
-    gated_scan_kernel<float><<<grid, dim3(256), 0, s>>>(gates, gate_b, u, decay, static_cast<const float*>(y),
-                                                       static_cast<const float*>(x), in_row, y_bias, x_bias,
-                                                       static_cast<float*>(out), state, state_row, item_start, slots,
-                                                       width, blocks, taps);
-  } else {
-    return fail("psamd_gated_scan: activation dtype must be float32 or bfloat16");
-  }
-  return check_launch("psamd_gated_scan");
+  if (act_dtype == kBF16)
+    return launch_scan<bf16_t>(s, gates, gate_b, u, decay, y, x, in_row, y_bias, x_bias, out, state, state_row, item_start, slots,
+                               items, tiles, n_tiles, tile, singles, n_singles, carry, width, blocks, taps);
+  if (act_dtype == kF32)
+    return launch_scan<float>(s, gates, gate_b, u, decay, y, x, in_row, y_bias, x_bias, out, state, state_row, item_start, slots,
+                              items, tiles, n_tiles, tile, singles, n_singles, carry, width, blocks, taps);
+  return fail("psamd_gated_scan: activation dtype must be float32 or bfloat16");
 }

@@ -50,7 +50,9 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
     ops.fixed_kv_len, ops.fixed_skew = runner.max_seq_len, ctx.decode_skewed
     try:
         # An eager run first: it sizes every workspace buffer (and is this step's result if
-        # capture is not possible). Then capture the same sequence and replay it.
+        # capture is not possible). Then capture the same sequence and replay it. Per-request
+        # state is saved first and put back before the replay, which applies the step a second time.
+        saved = {i: state.clone() for i, state in runner.states.items()}
         logits = runner.model.step(ctx)
         versions = (packer.version, ws.version)
         torch.cuda.synchronize(runner.device)
@@ -71,7 +73,9 @@ def graphed_decode_step(runner: "ModelRunner", items: Sequence[StepItem], token_
         if (packer.version, ws.version) != versions:
             return logits      # something grew during capture; try again on a later step
         runner._graphs[key] = (graph, captured, versions)
-        graph.replay()         # idempotent: same inputs, same cache writes as the eager run
+        for i, state in runner.states.items():
+            state.copy_(saved[i])
+        graph.replay()         # same inputs, same cache writes as the eager run
         return captured
     finally:
         ops.fixed_kv_len, ops.fixed_skew = previous

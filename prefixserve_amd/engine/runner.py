@@ -72,10 +72,11 @@ class ModelRunner:
         self.state_bytes_per_slot = sum(
             int(torch.empty((), dtype=n.dtype).element_size()) * int(torch.Size(n.shape).numel())
             for n in state_needs.values())
-        # A model whose mixers keep state of their own runs eagerly: capturing a step runs it
-        # once before and once after the capture, which pages of keys and values do not mind
-        # and a state that is added to does.
-        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and not state_needs
+        # Capturing a step runs it once before the capture and once as the first replay, which pages
+        # of keys and values do not mind and a state that is added to does: the capture saves and
+        # restores the state of mixers that allow it; a model with one that does not runs eagerly.
+        self.use_graphs = (bool(use_graphs) and self.device.type == "cuda"
+                           and (not state_needs or self.model.state_in_graphs()))
         self._graphs: dict[Any, Any] = {}
         if num_blocks is None:
             blocks = self._size_pools(reserve_bytes)

@@ -84,7 +84,8 @@ _SIGNATURES = {
     "psamd_heads_linear": [_vp, _vp, _i32, _i64, _i32, _vp, _i32, _vp, _i32, _i64, _i32, _i64, _i32, _i32, _i32],
     "psamd_latent_kv_append": [_vp, _vp, _i64, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _vp],
     "psamd_causal_conv": [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32],
-    "psamd_gated_scan": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32, _i32, _i32, _i32],
+    "psamd_gated_scan": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32,
+                         _vp, _i32, _i32, _vp, _i32, _vp, _i32, _i32, _i32],
     "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
     "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_moe_grouped_max_tiles": [_i64, _i32],
@@ -406,10 +407,19 @@ class HipOps:
         self._need(t == ctx.num_tokens, "gated_scan: token count differs from the step batch")
         sptr, srow = self._state_args(state, ctx, width, taps)
         size = rows.element_size()
+        # Items of more than one token are cut into the step's tiles of queries: summed up tile by tile,
+        # then run side by side. Room for the carries of the most tiles any step of this many tokens has.
+        n_tiles, n_single = int(ctx.num_prefill_tiles), int(ctx.num_decode)
+        self._need(ctx.pf_tiles.dtype == torch.int32 and ctx.dec_items.dtype == torch.int32, "gated_scan: the step's lists")
+        carry = None
+        if n_tiles:
+            carry = self.ws.get("recurrent.carry", (3 * n_tiles * width,), torch.float32)
         self._ok(self.lib.psamd_gated_scan(self._stream(), gates.data_ptr(), gate_bias.data_ptr(), u.data_ptr(), decay.data_ptr(),
                                            rows.data_ptr() + y_col * size, rows.data_ptr() + x_col * size, _code(rows.dtype),
                                            rows.shape[1], y_bias.data_ptr(), x_bias.data_ptr(), out.data_ptr(), sptr, srow,
-                                           ctx.item_start.data_ptr(), ctx.slots.data_ptr(), ctx.num_items, width, blocks, taps))
+                                           ctx.item_start.data_ptr(), ctx.slots.data_ptr(), ctx.num_items,
+                                           ctx.pf_tiles.data_ptr(), n_tiles, self.PREFILL_TILE_Q, ctx.dec_items.data_ptr(),
+                                           n_single, _ptr(carry), width, blocks, taps))
 
     def rope_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot) -> None:
         t = qkv.shape[0]

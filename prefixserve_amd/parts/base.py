@@ -203,6 +203,13 @@ class Mixer(Part):
     # tokens themselves); the block then lets the norm in front of it be lazy.
     takes_normed_rows = False
 
+    # For a mixer with state: True says that its kernels take slots and item boundaries from device
+    # memory and nothing from the host, so that a captured decode step serves every later step of
+    # its shape. The capture then saves the state before the step's eager run and puts it back
+    # before the first replay (the step would otherwise be applied to the state twice). A model
+    # with a stateful mixer that does not say so runs without captured steps.
+    state_in_graphs = False
+
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor | None:
         """x [T, hidden] (activation dtype) -> what is to be added to the residual: [T, hidden]

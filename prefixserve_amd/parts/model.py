@@ -125,6 +125,10 @@ class DecoderModel:
                 needs[i] = need
         return needs
 
+    def state_in_graphs(self) -> bool:
+        """Whether every mixer that keeps state lets a captured decode step update it."""
+        return all(blk.mixer.state_in_graphs for blk in self.blocks if blk.mixer.state_need() is not None)
+
     def attach(self, caches: Mapping[int, Any], states: Mapping[int, torch.Tensor]) -> None:
         self.caches = dict(caches)
         self.states = dict(states)

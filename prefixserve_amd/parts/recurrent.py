@@ -26,6 +26,8 @@ class GatedLinearRecurrence(Mixer):
     ``names``: "y", "y_bias", "x", "x_bias", "conv", "conv_bias", "gate_r", "gate_r_bias", "gate_i",
     "gate_i_bias", "lam", "o"."""
 
+    state_in_graphs = True
+
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], width: int, blocks: int, taps: int,
                  names: Mapping[str, str], decay_scale: float = 8.0) -> None:
         self.hidden_size, self.width, self.blocks, self.taps = int(hidden_size), int(width), int(blocks), int(taps)

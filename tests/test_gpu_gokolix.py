@@ -68,6 +68,11 @@ class Step:
         self.item_start = torch.tensor(starts, device=DEV)
         self.slots = torch.tensor(slots, dtype=torch.int32, device=DEV)
         self.tok_item = torch.tensor(np.repeat(np.arange(len(lengths)), lengths).astype(np.int32), device=DEV)
+        tiles = [(i, q) for i, n in enumerate(lengths) if n > 1 for q in range(0, n, 32)]
+        singles = [i for i, n in enumerate(lengths) if n == 1]
+        self.num_prefill_tiles, self.num_decode = len(tiles), len(singles)
+        self.pf_tiles = torch.tensor(np.asarray(tiles, dtype=np.int32).reshape(-1, 2), device=DEV)
+        self.dec_items = torch.tensor(np.asarray(singles, dtype=np.int32), device=DEV)
 
 
 # ------------------------------------------------------------------ kernels
@@ -210,7 +215,7 @@ def test_convolution_and_recurrence_continue_from_their_slot(ops, dtype, width, 
     wg, gb = rnd(blocks, 2 * bw, bw, seed=5, scale=0.4), rnd(blocks * 2 * bw, seed=6, scale=0.5)
     decay = -8.0 * torch.nn.functional.softplus(rnd(width, seed=7))
     state = torch.full((5, taps * width), 1e30, device=DEV)
-    seqs = {s: rnd(n, 2 * width, dtype=dtype, seed=10 + s) for s, n in ((4, 9), (1, 14), (2, 6), (0, 5))}
+    seqs = {s: rnd(n, 2 * width, dtype=dtype, seed=10 + s) for s, n in ((4, 109), (1, 14), (2, 70), (0, 5))}
 
     def plain_run(rows):                                   # one request, whole
         n = rows.shape[0]
@@ -239,9 +244,9 @@ def test_convolution_and_recurrence_continue_from_their_slot(ops, dtype, width, 
 
     for s in (4, 1, 2):
         state[s].zero_()                                   # what the runner does for a request at position 0
-    first = step([(4, seqs[4][:7]), (1, seqs[1][:3]), (2, seqs[2])])
+    first = step([(4, seqs[4][:7]), (1, seqs[1][:3]), (2, seqs[2])])           # the third is cut into three tiles
     state[0].zero_()
-    second = step([(1, seqs[1][3:4]), (0, seqs[0]), (4, seqs[4][7:])])
+    second = step([(1, seqs[1][3:4]), (0, seqs[0]), (4, seqs[4][7:])])         # the last continues over four tiles
     third = step([(1, seqs[1][4:])])
     got = {4: torch.cat([first[:7], second[6:]]), 1: torch.cat([first[7:10], second[:1], third]), 2: first[10:], 0: second[1:6]}
     tol = 2e-5 if dtype == torch.float32 else 2e-2
@@ -347,6 +352,34 @@ def test_decoding_through_graphs_without_a_recurrence(dtype, tmp_path):
     traces.compare(TraceReplayer(runner).run_step, steps, expect, [truth], 1.0, errors)
     check_rows(errors, dtype)
     assert runner._graphs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_through_graphs_with_a_recurrence(dtype, folders):
+    """The recurrence's kernels read slots and item boundaries from device memory, so its decode steps
+    are captured too; the capture puts the state back before its first replay. Two requests decode
+    side by side, then one alone (another graph), in slots that held junk."""
+    rng = np.random.default_rng(3)
+    reqs = [rng.integers(0, 96, n).tolist() for n in (60, 75)]
+    pm = plain.PlainGokolix(folders["A"])
+    truth = [pm.logits(t) for t in reqs]
+    runner = runner_for(folders["A"], 16, dtype, graphs=True)
+    assert runner.use_graphs and runner.states
+    for s in runner.states.values():
+        s.fill_(1e30)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": reqs[0][:20], "want": [19]}, {"id": "b", "tokens": reqs[1][:31], "want": [30]}], "end": []}]
+    expect = [[(0, 19), (1, 30)]]
+    for k in range(40):
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": [reqs[0][20 + k]], "want": [0]},
+                                                     {"id": "b", "tokens": [reqs[1][31 + k]], "want": [0]}], "end": ["a"] if k == 39 else []})
+        expect.append([(0, 20 + k), (1, 31 + k)])
+    for k in range(71, 75):
+        steps.append({"step": len(steps), "entries": [{"id": "b", "tokens": [reqs[1][k]], "want": [0]}], "end": ["b"] if k == 74 else []})
+        expect.append([(1, k)])
+    errors: list = []
+    traces.compare(TraceReplayer(runner).run_step, steps, expect, truth, 1.0, errors)
+    check_rows(errors, dtype)
+    assert len(runner._graphs) == 2
 
 
 def test_greedy_generation_through_the_entry_point(folders):
