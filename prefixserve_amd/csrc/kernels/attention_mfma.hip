@@ -1269,6 +1269,8 @@ static int launch_decode(hipStream_t s, const void* qkv, int q_stride, const voi
   const int group = hq / hkv;
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * 16 * NS);
   const int64_t groups_of_8 = ceil_div(static_cast<int64_t>(n_dec) * nsplit, 8);
+  if (!lds_allowed(attn_decode_mfma_kernel<NS, CT, P3>, smem))
+    return fail("psamd_attention_decode: " + std::to_string(smem) + " bytes of LDS were refused");
   attn_decode_mfma_kernel<NS, CT, P3><<<dim3(8 * hkv, static_cast<unsigned>(groups_of_8)), dim3(256), smem, s>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(kv), static_cast<bf16_t*>(out), part_o,
       part_ml, dec_items, item_start, item_end, table_off, block_ids, hq, hkv, nsplit, scale, window, min_tiles, n_dec,
@@ -1305,7 +1307,8 @@ int psamd_attention_mfma_supports(int hq, int hkv, int head_dim) {
   const bool dim_ok = head_dim % 16 == 0 && ((head_dim >= 16 && head_dim <= 128) || head_dim == 160 || head_dim == 192 ||
                                              head_dim == 256);
   const size_t smem = sizeof(float) * (8 * group + 4 * static_cast<size_t>(group) * head_dim);
-  return dim_ok && group <= 64 && smem <= 64 * 1024 && hq <= 65535 && hkv <= 65535;
+  // (the decode kernel's LDS: more than 64 KB is asked for at its launch, up to the 160 KB a compute unit has)
+  return dim_ok && group <= 64 && smem <= 160 * 1024 && hq <= 65535 && hkv <= 65535;
 }
 
 // Into how many runs psamd_attention_prefill may cut the keys of this step's query tiles; from 2

@@ -131,11 +131,25 @@ __global__ __launch_bounds__(256) void gated_scan_tiles_kernel(
   float* begin = carry + 2LL * n_tiles * width;                 // [n_tiles][width]: the item's starting state, at its first tile
   if (PASS == 0) {
     float P = 1.f, B = 0.f;
-    for (int64_t t = s0 + q0; t < s0 + q0 + n; ++t) {
-      float a, inflow;
-      scan_terms(gates[t * 2 * width + g_off] + br, gates[t * 2 * width + g_off + bw] + bi, dec, u[t * width + c], a, inflow);
-      B = fmaf(a, B, inflow);
-      P *= a;
+    // Eight tokens' operands are asked for together (they do not depend on the sums), then folded in order.
+    for (int64_t t8 = s0 + q0; t8 < s0 + q0 + n; t8 += 8) {
+      float gr[8], gi[8], uu[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int64_t t = min(t8 + i, s0 + q0 + n - 1);
+        gr[i] = gates[t * 2 * width + g_off];
+        gi[i] = gates[t * 2 * width + g_off + bw];
+        uu[i] = u[t * width + c];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (t8 + i < s0 + q0 + n) {
+          float a, inflow;
+          scan_terms(gr[i] + br, gi[i] + bi, dec, uu[i], a, inflow);
+          B = fmaf(a, B, inflow);
+          P *= a;
+        }
+      }
     }
     prod[static_cast<int64_t>(k) * width + c] = P;
     sum[static_cast<int64_t>(k) * width + c] = B;
@@ -146,11 +160,25 @@ __global__ __launch_bounds__(256) void gated_scan_tiles_kernel(
   float S = begin[static_cast<int64_t>(first) * width + c];
   for (int j = first; j < k; ++j) S = fmaf(prod[static_cast<int64_t>(j) * width + c], S, sum[static_cast<int64_t>(j) * width + c]);
   const float yb = y_bias[c];
-  for (int64_t t = s0 + q0; t < s0 + q0 + n; ++t) {
-    float a, inflow;
-    scan_terms(gates[t * 2 * width + g_off] + br, gates[t * 2 * width + g_off + bw] + bi, dec, u[t * width + c], a, inflow);
-    S = fmaf(a, S, inflow);
-    out[t * width + c] = from_float<A>(S * gelu_tanh_f(to_float<A>(y[t * in_row + c]) + yb));
+  for (int64_t t8 = s0 + q0; t8 < s0 + q0 + n; t8 += 8) {
+    float gr[8], gi[8], uu[8], yy[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t t = min(t8 + i, s0 + q0 + n - 1);
+      gr[i] = gates[t * 2 * width + g_off];
+      gi[i] = gates[t * 2 * width + g_off + bw];
+      uu[i] = u[t * width + c];
+      yy[i] = to_float<A>(y[t * in_row + c]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (t8 + i < s0 + q0 + n) {
+        float a, inflow;
+        scan_terms(gr[i] + br, gi[i] + bi, dec, uu[i], a, inflow);
+        S = fmaf(a, S, inflow);
+        out[(t8 + i) * width + c] = from_float<A>(S * gelu_tanh_f(yy[i] + yb));
+      }
+    }
   }
   if (q0 + n == len) {
     st[static_cast<int64_t>(taps - 1) * width + c] = S;

@@ -337,6 +337,19 @@ def test_long_contexts_without_windows(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_wide_latent_cache_entry(dtype, tmp_path):
+    """Sixteen heads on a cached vector of 192 + 64 = 256 numbers: the largest head the attention kernels
+    take, and more LDS in the decode kernel than a launch gets without asking."""
+    folder = write_gokolix(tmp_path, model(80, 64, 1e-5, 2.0, [layer(latent(16, 32, 64, 16, 192, 0.3, 10000.0, window=50), 32)]), seed=6)
+    toks = np.random.default_rng(5).integers(0, 80, 130).tolist()
+    truth = plain.PlainGokolix(folder).logits(toks)
+    steps, expect = traces.decode_tail([toks], tail=40)
+    errors: list = []
+    traces.compare(TraceReplayer(runner_for(folder, 12, dtype)).run_step, steps, expect, [truth], 1.0, errors)
+    check_rows(errors, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_through_graphs_without_a_recurrence(dtype, tmp_path):
     """A model of attention layers alone keeps no state, so its decode steps are captured: the
     replays give what single launches give."""
