@@ -89,11 +89,11 @@ class LatentAttention:
     @classmethod
     def from_json(cls, m: Mapping[str, Any], where: str) -> "LatentAttention":
         _only(m, ("heads", "dim", "rot_dim", "vdim", "kv_rank", "scale", "rot", "mask"), where)
-        rot = m["rot"]
+        rot_dim = int(m.get("rot_dim", 0))
+        rot = m.get("rot") or {"base": 10000.0, "dims": rot_dim}       # a mixer without a rotated part need not describe a rotation
         _only(rot, ("base", "dims", "scaling"), where + ".rot")
-        rot_dim = int(m["rot_dim"])
-        if int(rot["dims"]) != rot_dim or rot_dim % 2 or rot_dim < 0:
-            raise UnsupportedModelError(f"{where}: the rotated part is rot_dim = {rot_dim} wide and even; rot.dims says {rot['dims']}")
+        if int(rot.get("dims", rot_dim)) != rot_dim or rot_dim % 2 or rot_dim < 0:
+            raise UnsupportedModelError(f"{where}: the rotated part is rot_dim = {rot_dim} wide and even; rot.dims says {rot.get('dims')}")
         if int(m["heads"]) < 1 or int(m["kv_rank"]) < 1:
             raise UnsupportedModelError(f"{where}: heads and kv_rank must be positive")
         return cls(int(m["heads"]), int(m["dim"]), rot_dim, int(m["vdim"]), int(m["kv_rank"]), float(m["scale"]),
