@@ -1,6 +1,6 @@
 // Causal grouped-query attention over the paged cache, the straightforward way: one wave
-// per (new token, query head), float arithmetic throughout, any head size that is a
-// multiple of 2 up to 256, any number of heads and groups, optional sliding window, an optional
+// per (new token, query head), float arithmetic throughout, any head size up to 512, any number
+// of heads and groups, optional sliding window, an optional
 // learned sink per head (a term exp(sink) in the softmax's denominator that has no key and no
 // value) and an optional bias on the scaled score that depends on the head and on how far back
 // the key lies (a table per head, its last entry standing for every larger distance).
@@ -15,6 +15,8 @@
 
 namespace psamd {
 
+constexpr int kMaxHead = 512;          // head sizes up to here: kMaxHead / 64 output dimensions per lane
+
 template <typename A>
 __global__ __launch_bounds__(64) void attention_generic_kernel(
     const A* __restrict__ qkv, int q_stride, A* __restrict__ out, const A* __restrict__ kv,
@@ -22,7 +24,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int32_t* __restrict__ table_off, const int32_t* __restrict__ block_ids,
     int hq, int hkv, int d, float scale, int window, const float* __restrict__ sink,
     const float* __restrict__ dist_bias, int n_dist) {
-  __shared__ float q_s[256];
+  __shared__ float q_s[kMaxHead];
   __shared__ float p_s[kWave];
   __shared__ int32_t base_s[kWave];   // element offset of (page, kv head) for each key of the chunk
   __shared__ int32_t off_s[kWave];
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};   // dims lane, lane+64, lane+128, lane+192
+  float acc[kMaxHead / kWave] = {};      // dims lane, lane+64, lane+128, ...
   for (int c0 = k_lo; c0 <= pos; c0 += kWave) {
     const int j = c0 + lane;
     float s = -INFINITY;
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     __syncthreads();
     const int cnt = min(kWave, pos - c0 + 1);
 #pragma unroll
-    for (int dd = 0; dd < 4; ++dd) {
+    for (int dd = 0; dd < kMaxHead / kWave; ++dd) {
       const int i = lane + dd * kWave;
       if (i < d) {
         float a = acc[dd] * alpha;
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   const float inv = 1.f / l;
   A* o = out + t * (static_cast<int64_t>(hq) * d) + h * d;
 #pragma unroll
-  for (int dd = 0; dd < 4; ++dd) {
+  for (int dd = 0; dd < kMaxHead / kWave; ++dd) {
     const int i = lane + dd * kWave;
     if (i < d) o[i] = from_float<A>(acc[dd] * inv);
   }
@@ -102,7 +104,7 @@ extern "C" int psamd_attention_generic(void* stream, const void* qkv, int q_stri
                                        const float* dist_bias, int n_dist) {
   PSAMD_REQUIRE(dist_bias == nullptr || n_dist >= 1, "a distance bias needs at least one entry per head");
   PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv > 0 && hq % hkv == 0, "bad head counts");
-  PSAMD_REQUIRE(head_dim > 0 && head_dim <= 256, "head_dim must be in [1, 256]");
+  PSAMD_REQUIRE(head_dim > 0 && head_dim <= kMaxHead, "head_dim must be in [1, 512]");
   PSAMD_REQUIRE(hq <= 65535, "too many heads for one launch");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -28,14 +28,16 @@ class LayerCache:
     window: int | None
 
 
-def slot_size(head_dim: int, value_dim: int) -> int:
+def slot_size(head_dim: int, value_dim: int, largest: int = 256) -> int:
     """The head size the pages and kernels run with: the larger of the two sizes, rounded up to
-    one the matrix-core attention takes (multiples of 16 up to 128, then 160, 192, 256)."""
+    one the matrix-core attention takes (multiples of 16 up to 128, then 160, 192, 256). A mixer
+    whose other kernels take more may allow up to 512 (``largest``): sizes above 256 are multiples
+    of 64 and run the attention kernel of the 32-bit path in either dtype."""
     need = max(int(head_dim), int(value_dim))
-    for size in (*range(16, 129, 16), 160, 192, 256):
-        if need <= size:
+    for size in (*range(16, 129, 16), 160, 192, 256, 320, 384, 448, 512):
+        if need <= size <= largest:
             return size
-    raise ValueError(f"head sizes up to 256 are implemented, got {need}")
+    raise ValueError(f"head sizes up to {largest} are implemented, got {need}")
 
 
 def head_slots(head_dim: int, rotary_dim: int, slots: int) -> list[int]:

@@ -48,7 +48,7 @@ class LatentAttention(Mixer):
             if not isinstance(self.pos, RotaryTable) or self.pos.head_dim != self.rot_dim \
                     or (self.pos.rotary_dim or self.rot_dim) != self.rot_dim:
                 raise ValueError(f"the rotated part needs a rotation table of {self.rot_dim} dimensions")
-        self.slots = slot_size(self.rank + self.rot_dim, self.rank)
+        self.slots = slot_size(self.rank + self.rot_dim, self.rank, largest=512)
         self.q_width = self.num_heads * (self.head_dim + self.rot_dim)
 
     def weights(self) -> dict[str, WeightWant]:

@@ -350,6 +350,18 @@ def test_a_wide_latent_cache_entry(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_latent_cache_entry_wider_than_the_matrix_core_kernels_take(dtype, tmp_path):
+    """288 + 40 = 328 numbers per token: a 384-wide entry, served by the 32-bit path's attention kernel."""
+    folder = write_gokolix(tmp_path, model(80, 64, 1e-5, 2.0, [layer(latent(3, 24, 40, 16, 288, 0.3, 10000.0, window=30), 32)]), seed=7)
+    toks = np.random.default_rng(5).integers(0, 80, 75).tolist()
+    truth = plain.PlainGokolix(folder).logits(toks)
+    steps, expect = traces.decode_tail([toks], tail=20)
+    errors: list = []
+    traces.compare(TraceReplayer(runner_for(folder, 8, dtype)).run_step, steps, expect, [truth], 1.0, errors)
+    check_rows(errors, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_through_graphs_without_a_recurrence(dtype, tmp_path):
     """A model of attention layers alone keeps no state, so its decode steps are captured: the
     replays give what single launches give."""
